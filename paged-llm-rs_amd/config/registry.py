@@ -9,6 +9,7 @@ from __future__ import annotations
 from pathlib import Path
 
 from ..errors import ConfigError, UnsupportedError
+from .papivik import PapivikConfig
 from .qwen3 import Qwen3Config, read_json
 
 _ARCHITECTURES: dict = {}
@@ -30,6 +31,8 @@ def config_class_for(d: dict):
     if not isinstance(d, dict):
         raise ConfigError("config.json does not hold an object")
     names = d.get("architectures")
+    if names is None and isinstance(d.get("architecture"), str):
+        names = [d["architecture"]]            # (a config.json that names its one architecture in the singular)
     if isinstance(names, list) and names:
         name = names[0]
         if isinstance(name, str) and name in _ARCHITECTURES:
@@ -60,3 +63,4 @@ def load_config(source):
 
 
 register_architecture("Qwen3ForCausalLM", Qwen3Config, model_type="qwen3")
+register_architecture("Papivik", PapivikConfig, model_type="papivik")

@@ -94,3 +94,73 @@ class ModelSpec:
     # a learned position added to it), ``extra["logit_transform"]`` to the 32-bit logits (a soft cap, a
     # scale).  Each transform reads its own constants from ``extra`` too.  None of the two by default.
     extra: dict = field(default_factory=dict)
+
+
+# ---- mixers that carry a state from token to token, and layers built around them --------------------
+
+@dataclass(frozen=True)
+class LinearAttentionSpec:
+    """Linear attention with one fixed decay a head: S = decay S + k v^T, o = S^T q, with q, k and v through
+    silu; the read-out normalised over all heads together, times sigmoid(gate)."""
+    kind: str = "lightning_attention"
+    num_heads: int = 0
+    head_dim: int = 0            # size of q and k a head
+    value_dim: int = 0           # size of v a head
+    decay: tuple = ()            # one a head
+    eps: float = 1e-6
+
+
+@dataclass(frozen=True)
+class MlstmSpec:
+    """A matrix memory a head with exponential input and forget gates, held stable by a running maximum."""
+    kind: str = "mlstm"
+    num_heads: int = 0
+    head_dim: int = 0
+    value_dim: int = 0
+    gate_cap: float = 15.0       # the gates' pre-activations pass cap * tanh(x / cap)
+    eps: float = 1e-6
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """The gated delta rule: S = g S; S += k (beta (v - S^T k))^T; o = S^T q, behind short convolutions."""
+    kind: str = "gated_delta"
+    num_heads: int = 0           # heads of v
+    num_qk_heads: int = 0        # heads of q and k (divides num_heads)
+    head_dim: int = 0
+    value_dim: int = 0
+    conv_taps: int = 4
+    eps: float = 1e-6
+
+
+@dataclass(frozen=True)
+class ConvAttentionSpec:
+    """Grouped-query softmax attention over a paged cache whose q, k and v pass a short causal convolution
+    right behind their projections; value heads may have another size than query and key heads."""
+    kind: str = "conv_attention"
+    num_heads: int = 0
+    num_kv_heads: int = 0
+    head_dim: int = 0
+    value_dim: int = 0
+    conv_taps: int = 1
+    qk_norm_eps: Optional[float] = None     # None: no norm a head on q and k
+    rotary_dim: int = 0                     # how many values of a head turn (0: none)
+    rotary_base: float = 10000.0
+    scale: Optional[float] = None           # None = 1/sqrt(head_dim)
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class ParallelMixersSpec:
+    """Several mixers that read the same rows; their outputs are added with a weight each.
+    ``branches``: ((tensor-name part, mixer spec, weight), ...)."""
+    kind: str = "parallel_mixers"
+    branches: tuple = ()
+
+
+@dataclass(frozen=True)
+class DenseMlpSpec:
+    """down(act(up(x)))."""
+    kind: str = "dense_mlp"
+    intermediate_size: int = 0
+    activation: str = "gelu_tanh"

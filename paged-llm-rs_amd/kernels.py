@@ -53,6 +53,18 @@ def _signatures(lib) -> None:
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
         "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, i, p],
         "pl_paged_attention_grouped_applies": [i, i, i, i],
+        "pl_recurrent_scan": [i, p, i, i, i, i, p, i, i, i, p, p, f, p, ctypes.c_long, i, i, i, p, p, p, p,
+                              i, i, i, i, i, p],
+        "pl_short_conv": [p, i, i, i, p, i, p, ctypes.c_long, i, p, p, p, p, p, i, i, p],
+        "pl_conv_history": [p, i, i, i, i, p, ctypes.c_long, i, p, p, p, i, p],
+        "pl_gated_group_norm": [p, i, i, i, p, i, f, p, i, i, i, p, i, p],
+        "pl_conv_qk_prepare": [p, i, i, p, i, p, ctypes.c_long, i, p, p, f, p, i, p, p, p, p, p, i, i, p, p, p, i,
+                               i, i, i, i, i, i, p],
+        "pl_rmsnorm_onto": [p, p, p, f, p, i, i, i, p],
+        "pl_scale": [p, f, ctypes.c_long, p],
+        "pl_to_bf16": [p, p, ctypes.c_long, p],
+        "pl_activation": [p, p, i, i, ctypes.c_long, p],
+        "pl_weighted_sum": [p, f, p, f, ctypes.c_long, p],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name)
@@ -1026,3 +1038,216 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype,
     if splits > 1:
         return gemm_split_library(x, w, splits, out_dtype)
     return torch.mm(x, w.t())
+
+
+# ---------------------------------------------------------------------------
+# Mixers with a carried state, short convolutions, and the layer that normalises a sublayer's output
+
+SCAN_KINDS = {"lightning": 0, "mlstm": 1, "delta": 2}
+SCAN_MAX_DIM = 256
+
+
+def _state_view(state: torch.Tensor, what: str):
+    """(tensor, floats between two slots): a [slots, floats] 32-bit state, possibly a run of columns of a wider one."""
+    if not isinstance(state, torch.Tensor) or not state.is_cuda or state.dtype != torch.float32 or state.dim() != 2 \
+            or (state.shape[1] > 0 and state.stride(1) != 1):
+        raise TensorError(f"{what} is not a 32-bit [slots, floats] tensor on the GPU with unit stride along a slot")
+    return state, state.stride(0)
+
+
+def _step_rows(batch, n: int):
+    for t, what, count in ((batch.q_start, "first rows", batch.num_seqs), (batch.q_len, "row counts", batch.num_seqs),
+                           (batch.state_slots, "state slots", batch.num_seqs), (batch.positions, "positions", n),
+                           (batch.seq_of, "request index of each token", n)):
+        _need(t, what, (count,), torch.int32)
+
+
+def recurrent_scan(kind: str, qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, state: torch.Tensor,
+                   batch, heads: int, qk_heads: int, dim: int, vdim: int, *, gates: torch.Tensor | None = None,
+                   g1_off: int = 0, g2_off: int = 0, p1: torch.Tensor | None = None, p2: torch.Tensor | None = None,
+                   cap: float = 0.0, out: torch.Tensor | None = None) -> torch.Tensor:
+    """The read-out [rows, heads * vdim] (32-bit) of a mixer that carries a [dim, vdim] matrix a head from
+    token to token, over the tokens of a step, request by request, from and into the requests' state slots.
+
+    ``lightning``: S = decay S + silu(k) silu(v)^T, o = S^T silu(q); ``p1`` = the decays.
+    ``mlstm``: log gates i = cap tanh((x1 + b_i)/cap), f = logsigmoid(cap tanh((x2 + b_f)/cap)) from the two
+    gate columns a head, a running maximum m, S and a normaliser n; ``p1``, ``p2`` = the biases; the state a
+    slot is S [heads, dim, vdim], n [heads, dim], m [heads].
+    ``delta``: ``qkv`` holds convolved and activated rows; q and k become unit vectors, beta = sigmoid(x1),
+    decay = exp(-exp(A_log) softplus(x2 + dt_bias)); ``p1`` = A_log, ``p2`` = dt_bias.
+    q and k have ``qk_heads`` heads (head h of v reads head h / (heads / qk_heads))."""
+    if kind not in SCAN_KINDS:
+        raise TensorError(f"a scan of kind {kind!r}, the kernels know {', '.join(SCAN_KINDS)}")
+    n = qkv.shape[0]
+    _need(qkv, "rows of q, k and v", None, torch.float32)
+    if qkv.dim() != 2:
+        raise TensorError(f"rows of q, k and v of shape {tuple(qkv.shape)}")
+    width = qkv.shape[1]
+    if not (0 <= q_off and q_off + qk_heads * dim <= width and 0 <= k_off and k_off + qk_heads * dim <= width
+            and 0 <= v_off and v_off + heads * vdim <= width):
+        raise TensorError(f"q, k, v at columns {q_off}, {k_off}, {v_off} of rows of {width}")
+    if heads < 1 or qk_heads < 1 or heads % qk_heads or not 1 <= dim <= SCAN_MAX_DIM or vdim < 1:
+        raise TensorError(f"a scan over {heads} heads ({qk_heads} of q and k) of {dim} by {vdim}")
+    state, stride = _state_view(state, "the state")
+    need = heads * dim * vdim + (heads * dim + heads if kind == "mlstm" else 0)
+    if state.shape[1] != need:
+        raise TensorError(f"a state of {state.shape[1]} floats a slot, this mixer keeps {need}")
+    _step_rows(batch, n)
+    if kind != "lightning":
+        _need(gates, "rows of the gates", None, torch.float32)
+        if gates.dim() != 2 or gates.shape[0] != n or not (0 <= g1_off and g1_off + heads <= gates.shape[1]
+                                                         and 0 <= g2_off and g2_off + heads <= gates.shape[1]):
+            raise TensorError(f"gates at columns {g1_off}, {g2_off} of rows of shape {tuple(gates.shape)}")
+        _need(p2, "second gate constant", (heads,), torch.float32)
+    _need(p1, "decays" if kind == "lightning" else "first gate constant", (heads,), torch.float32)
+    if out is None:
+        out = torch.empty((n, heads * vdim), dtype=torch.float32, device=qkv.device)
+    _need(out, "read-out", (n, heads * vdim), torch.float32)
+    hdv = heads * dim * vdim
+    _check(library().pl_recurrent_scan(
+        SCAN_KINDS[kind], qkv.data_ptr(), width, q_off, k_off, v_off, _ptr(gates),
+        0 if gates is None else gates.shape[1], g1_off, g2_off, _ptr(p1), _ptr(p2), float(cap),
+        state.data_ptr(), stride, 0, hdv, hdv + heads * dim, out.data_ptr(), batch.q_start.data_ptr(),
+        batch.q_len.data_ptr(), batch.state_slots.data_ptr(), batch.num_seqs, heads, qk_heads, dim, vdim, _stream()))
+    return out
+
+
+def _conv_args(rows, off, weight, history, batch):
+    n = rows.shape[0]
+    _need(rows, "projected rows", None, torch.float32)
+    _need(weight, "convolution filters", None, torch.float32)
+    if rows.dim() != 2 or weight.dim() != 2:
+        raise TensorError(f"rows of shape {tuple(rows.shape)}, filters of shape {tuple(weight.shape)}")
+    channels, taps = weight.shape
+    if not 1 <= taps <= 16 or off < 0 or off + channels > rows.shape[1]:
+        raise TensorError(f"{channels} channels of {taps} taps from column {off} of rows of {rows.shape[1]}")
+    history, stride = _state_view(history, "the convolution's history")
+    if history.shape[1] != (taps - 1) * channels:
+        raise TensorError(f"a history of {history.shape[1]} floats a slot for {taps} taps over {channels} channels")
+    _step_rows(batch, n)
+    return n, channels, taps, history, stride
+
+
+def short_conv(rows: torch.Tensor, off: int, weight: torch.Tensor, history: torch.Tensor, batch,
+               silu: bool = False, out: torch.Tensor | None = None) -> torch.Tensor:
+    """y[t, c] = sum_j weight[c, j] * u[t - taps + 1 + j, c] over the columns [off, off + channels) of
+    ``rows``; the rows before a request's first of this step come from ``history`` [slots, (taps-1) * channels]
+    (newest last, zeros at a request's start), which is left as it is: ``conv_history`` moves it afterwards."""
+    n, channels, taps, history, stride = _conv_args(rows, off, weight, history, batch)
+    if out is None:
+        out = torch.empty((n, channels), dtype=torch.float32, device=rows.device)
+    _need(out, "convolved rows", (n, channels), torch.float32)
+    _check(library().pl_short_conv(rows.data_ptr(), rows.shape[1], off, channels, weight.data_ptr(), taps,
+                                   history.data_ptr(), stride, 0, batch.positions.data_ptr(), batch.seq_of.data_ptr(),
+                                   batch.q_start.data_ptr(), batch.state_slots.data_ptr(), out.data_ptr(),
+                                   1 if silu else 0, n, _stream()))
+    return out
+
+
+def conv_history(rows: torch.Tensor, off: int, weight: torch.Tensor, history: torch.Tensor, batch) -> None:
+    """The history becomes the last taps - 1 inputs of every request of the step."""
+    n, channels, taps, history, stride = _conv_args(rows, off, weight, history, batch)
+    _check(library().pl_conv_history(rows.data_ptr(), rows.shape[1], off, channels, taps, history.data_ptr(), stride, 0,
+                                     batch.q_start.data_ptr(), batch.q_len.data_ptr(), batch.state_slots.data_ptr(),
+                                     batch.num_seqs, _stream()))
+
+
+GATES = {None: -1, "sigmoid": 0, "silu": 1}
+
+
+def gated_group_norm(x: torch.Tensor, group: int, gain: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                     gate: torch.Tensor | None = None, gate_off: int = 0, gate_act: str | None = None) -> torch.Tensor:
+    """x / sqrt(mean over each run of ``group`` columns of x^2 + eps) * gain * act(gate); ``gain`` has a value a
+    column or a value a column of a group; ``gate`` are the columns from ``gate_off`` of 32-bit rows."""
+    n, width = x.shape
+    _need(x, "read-out", None, torch.float32)
+    _need(gain, "gain of the grouped norm", None, torch.float32)
+    if group < 1 or width % group or gain.numel() not in (group, width):
+        raise TensorError(f"rows of {width} in groups of {group} with {gain.numel()} gains")
+    if gate_act not in GATES or (gate_act is None) != (gate is None):
+        raise TensorError(f"a gate through {gate_act!r}")
+    if gate is not None:
+        _need(gate, "rows of the gate", None, torch.float32)
+        if gate.dim() != 2 or gate.shape[0] != n or gate_off < 0 or gate_off + width > gate.shape[1]:
+            raise TensorError(f"a gate at column {gate_off} of rows of shape {tuple(gate.shape)}")
+    out = torch.empty((n, width), dtype=out_dtype, device=x.device)
+    _check(library().pl_gated_group_norm(x.data_ptr(), n, width, group, gain.data_ptr(), gain.numel(), float(eps),
+                                         _ptr(gate), 0 if gate is None else gate.shape[1], gate_off, GATES[gate_act],
+                                         out.data_ptr(), _code(out, "normalised read-out"), _stream()))
+    return out
+
+
+def conv_qk_prepare(rows: torch.Tensor, off: int, weight: torch.Tensor, history: torch.Tensor, q_gain, k_gain,
+                    eps: float, freq, rot: int, batch, kv, heads: int, kv_heads: int, dim: int, vdim: int,
+                    padded: int, q_out: torch.Tensor) -> torch.Tensor:
+    """For an attention layer with short convolutions: convolution of the projected q | k | v columns, norm a
+    head of q and k, rotation of the first ``rot`` values of a head by position * freq, q into ``q_out``
+    [rows, heads * padded] and k, v into the pages, every head in a row of ``padded`` values."""
+    n, channels, taps, history, stride = _conv_args(rows, off, weight, history, batch)
+    if channels != heads * dim + kv_heads * dim + kv_heads * vdim:
+        raise TensorError(f"{channels} channels for {heads} heads and {kv_heads} key heads of {dim} and {vdim}")
+    _need(q_gain, "query norm gain", (dim,), torch.float32)
+    _need(k_gain, "key norm gain", (dim,), torch.float32)
+    if rot:
+        _need(freq, "rotation frequencies", (rot // 2,), torch.float32)
+    if rot < 0 or rot % 2 or rot > dim or not max(dim, vdim) <= padded <= 256:
+        raise TensorError(f"a rotation over {rot} of {dim} values, heads in rows of {padded}")
+    _need(q_out, "query buffer", (n, heads * padded))
+    for pool, what in ((kv.k_pool, "key pool"), (kv.v_pool, "value pool")):
+        _need(pool, what, None, q_out.dtype)
+        if pool.dim() != 2 or pool.shape[1] != kv_heads * padded or pool.shape[0] % kv.block_size:
+            raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{kv.block_size}, {kv_heads * padded}]")
+    _need(kv.block_table, "block table", None, torch.int32)
+    if kv.block_table.dim() != 2 or kv.block_table.shape[0] != batch.num_seqs:
+        raise TensorError(f"block table has shape {tuple(kv.block_table.shape)} for {batch.num_seqs} requests")
+    _check(library().pl_conv_qk_prepare(
+        rows.data_ptr(), rows.shape[1], off, weight.data_ptr(), taps, history.data_ptr(), stride, 0,
+        q_gain.data_ptr(), k_gain.data_ptr(), float(eps), _ptr(freq) if rot else 0, rot,
+        batch.positions.data_ptr(), batch.seq_of.data_ptr(), batch.q_start.data_ptr(), batch.state_slots.data_ptr(),
+        kv.block_table.data_ptr(), kv.block_table.shape[1], kv.block_size, q_out.data_ptr(), kv.k_pool.data_ptr(),
+        kv.v_pool.data_ptr(), _code(q_out, "query buffer"), n, heads, kv_heads, dim, vdim, padded, _stream()))
+    return q_out
+
+
+def rmsnorm_onto(resid: torch.Tensor, y: torch.Tensor, gain: torch.Tensor, eps: float,
+                 rows_dtype: torch.dtype | None = None):
+    """resid += y / sqrt(mean(y^2) + eps) * gain, all 32-bit.  With ``rows_dtype`` the updated rows come back
+    in that type as well (what the next part multiplies), otherwise None."""
+    n, H = resid.shape
+    _need(resid, "residual stream", None, torch.float32)
+    _need(y, "sublayer output", (n, H), torch.float32)
+    _need(gain, "norm gain", (H,), torch.float32)
+    rows = None if rows_dtype is None else torch.empty((n, H), dtype=rows_dtype, device=resid.device)
+    _check(library().pl_rmsnorm_onto(resid.data_ptr(), y.data_ptr(), gain.data_ptr(), float(eps), _ptr(rows),
+                                     F32 if rows is None else _code(rows, "rows of the stream"), n, H, _stream()))
+    return rows
+
+
+def scale_(x: torch.Tensor, s: float) -> torch.Tensor:
+    _need(x, "values to scale", None, torch.float32)
+    _check(library().pl_scale(x.data_ptr(), float(s), x.numel(), _stream()))
+    return x
+
+
+def to_bf16(x: torch.Tensor) -> torch.Tensor:
+    _need(x, "32-bit rows", None, torch.float32)
+    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    _check(library().pl_to_bf16(x.data_ptr(), out.data_ptr(), x.numel(), _stream()))
+    return out
+
+
+def activation(x: torch.Tensor, name: str) -> torch.Tensor:
+    """act(x) element by element, computed in 32-bit and rounded once."""
+    _need(x, "values to activate")
+    out = torch.empty_like(x)
+    _check(library().pl_activation(x.data_ptr(), out.data_ptr(), _code(x, "values to activate"), activation_code(name),
+                                   x.numel(), _stream()))
+    return out
+
+
+def weighted_sum_(x: torch.Tensor, a: float, y: torch.Tensor, b: float) -> torch.Tensor:
+    """x = a x + b y, 32-bit."""
+    _need(x, "first branch", None, torch.float32)
+    _need(y, "second branch", tuple(x.shape), torch.float32)
+    _check(library().pl_weighted_sum(x.data_ptr(), float(a), y.data_ptr(), float(b), x.numel(), _stream()))
+    return x

@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import torch
 
+from .. import kernels
 from ..errors import ConfigError
 from .norm import PendingNorm
 from .registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, lookup, prefixed, register_block, scoped)
@@ -126,3 +127,77 @@ class PreNormBlock:
 
 
 register_block("pre_norm", PreNormBlock)
+
+
+class SublayerNormBlock:
+    """The arrangement that normalises what a sublayer gives instead of what it gets:
+    x <- x + norm1(mixer(x)), then x <- x + norm2(feed_forward(x)); the sublayers read the stream itself.
+    A layer whose spec has no feed-forward has the first sublayer only.
+
+    The stream is 32-bit; the parts multiply its rows in the model's type, which the norm kernel that
+    updates the stream leaves behind for the next part (``ctx.stream_rows`` carries them from layer to
+    layer).  Mixers and feed-forwards hand back 32-bit rows, the unrounded sums of their last product.
+    Tensor names: the norms' gains are stored under the norms' own names."""
+
+    NAMES = {"norm1": "norm1", "mixer": "mix", "norm2": "norm2", "feed_forward": "mlp"}
+
+    @classmethod
+    def names_of(cls, layer) -> dict:
+        given = getattr(layer, "names", None) or {}
+        unknown = sorted(set(given) - set(cls.NAMES))
+        if unknown:
+            raise ConfigError(f"a layer names members that this arrangement does not have: {unknown}")
+        return {**cls.NAMES, **given}
+
+    @classmethod
+    def declare(cls, layer, hidden: int) -> list:
+        from ..weights.loader import ParamDecl
+
+        n = cls.names_of(layer)
+        mixer = lookup(MIXERS, layer.mixer.kind, "mixer")
+        decls = [ParamDecl(n["norm1"], (hidden,), "gain")] + prefixed(mixer.declare(layer.mixer, hidden), n["mixer"])
+        if layer.feed_forward is not None:
+            ffn = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")
+            decls += [ParamDecl(n["norm2"], (hidden,), "gain")] + prefixed(ffn.declare(layer.feed_forward, hidden), n["feed_forward"])
+        return decls
+
+    def __init__(self, layer, hidden: int, params: dict, dtype, device, shared: dict):
+        n = self.names = self.names_of(layer)
+        norm = lookup(NORMS, layer.norm.kind, "norm")
+        if not hasattr(norm, "apply_onto"):
+            raise ConfigError(f"norm {layer.norm.kind!r} cannot normalise a sublayer's output onto the stream")
+        self.dtype = dtype
+        self.norm1 = norm(layer.norm, hidden, {"weight": params[n["norm1"]]}, dtype, device)
+        self.mixer = lookup(MIXERS, layer.mixer.kind, "mixer")(
+            layer.mixer, hidden, scoped(params, n["mixer"]), dtype, device, shared)
+        self.norm2 = self.feed_forward = None
+        if layer.feed_forward is not None:
+            self.norm2 = norm(layer.norm, hidden, {"weight": params[n["norm2"]]}, dtype, device)
+            self.feed_forward = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")(
+                layer.feed_forward, hidden, scoped(params, n["feed_forward"]), dtype, device, shared)
+
+    @property
+    def graph_safe(self) -> bool:
+        return getattr(self.mixer, "graph_safe", True) and getattr(self.feed_forward, "graph_safe", True)
+
+    def _rows(self, resid, ctx):
+        """The stream's rows in the model's type: what the part before left, or a pass of their own."""
+        if self.dtype == torch.float32:
+            return resid
+        rows = getattr(ctx, "stream_rows", None)
+        return rows if rows is not None else kernels.to_bf16(resid)
+
+    def forward(self, resid, delta, ctx):
+        if delta is not None:
+            kernels.residual_add(resid, delta)
+            ctx.stream_rows = None
+        rows_dtype = None if self.dtype == torch.float32 else self.dtype
+        mixed = self.mixer.forward(self._rows(resid, ctx), ctx)
+        ctx.stream_rows = self.norm1.apply_onto(resid, mixed, rows_dtype)
+        if self.feed_forward is not None:
+            out = self.feed_forward.forward(self._rows(resid, ctx))
+            ctx.stream_rows = self.norm2.apply_onto(resid, out, rows_dtype)
+        return None
+
+
+register_block("sublayer_norm", SublayerNormBlock)

@@ -54,3 +54,26 @@ class GatedMlp:
 
 
 register_feed_forward("gated_mlp", GatedMlp)
+
+
+class DenseMlp:
+    """down(act(up(x))): two products with an activation between them.  The result comes back in 32-bit
+    (the sums of the second product, unrounded) for a layer that normalises it before it joins the stream."""
+
+    @staticmethod
+    def declare(spec, hidden: int) -> list:
+        return [ParamDecl("up", (spec.intermediate_size, hidden)), ParamDecl("down", (hidden, spec.intermediate_size))]
+
+    def __init__(self, spec, hidden: int, params: dict, dtype, device, shared: dict):
+        if spec.activation not in kernels.ACTIVATIONS:
+            raise UnsupportedError(f"activation {spec.activation!r}, the kernels know {', '.join(sorted(kernels.ACTIVATIONS))}")
+        self.activation = spec.activation
+        self.up_proj = Linear(params["up"])
+        self.down_proj = Linear(params["down"])
+
+    def forward(self, x):
+        return self.down_proj.forward(kernels.activation(self.up_proj.forward(x), self.activation),
+                                      out_dtype=torch.float32)
+
+
+register_feed_forward("dense_mlp", DenseMlp)

@@ -16,7 +16,7 @@ from ..cache.layout import CacheLayout
 from ..config import load_config
 from ..errors import ConfigError, UnsupportedError, WeightError
 from ..weights.loader import ParamDecl, load_weights
-from . import attention, block, mlp, norm  # noqa: F401  (register the built-in parts)
+from . import attention, block, conv_attention, mlp, norm, parallel, recurrent, transforms  # noqa: F401  (register the built-in parts)
 from .linear import Linear, linears_of
 from .norm import PendingNorm
 from .registry import BLOCKS, EMBED_TRANSFORMS, LOGIT_TRANSFORMS, NORMS, lookup, prefixed, scoped
@@ -37,6 +37,23 @@ def _transforms(spec) -> list:
     return found
 
 
+def _final_norm_decls(spec, final) -> list:
+    """The final norm's tensors: under the stem of ``final_norm_name``, or, where the spec says that a norm's
+    gain is stored under the norm's own name (``extra["bare_norm_names"]``), the one tensor of that name."""
+    if (spec.extra or {}).get("bare_norm_names"):
+        decls = final.declare(spec.final_norm, spec.hidden_size)
+        if len(decls) != 1:
+            raise ConfigError(f"a norm of {len(decls)} tensors cannot be stored under its own name alone")
+        return [ParamDecl(spec.final_norm_name, decls[0].shape, decls[0].role, decls[0].optional)]
+    return prefixed(final.declare(spec.final_norm, spec.hidden_size), spec.final_norm_name.rsplit(".", 1)[0])
+
+
+def _final_norm_params(spec, final, params: dict) -> dict:
+    if (spec.extra or {}).get("bare_norm_names"):
+        return {final.declare(spec.final_norm, spec.hidden_size)[0].name: params[spec.final_norm_name]}
+    return scoped(params, spec.final_norm_name.rsplit(".", 1)[0])
+
+
 def declare_parameters(spec) -> list:
     """Every tensor the model needs, by checkpoint name (reference: model/mod.rs:178-227)."""
     decls = [ParamDecl(spec.embed_name, (spec.vocab_size, spec.hidden_size), "embedding")]
@@ -44,8 +61,7 @@ def declare_parameters(spec) -> list:
         cls = lookup(BLOCKS, layer.block, "block")
         decls += prefixed(cls.declare(layer, spec.hidden_size), layer.weight_prefix)
     final = lookup(NORMS, spec.final_norm.kind, "norm")
-    stem = spec.final_norm_name.rsplit(".", 1)[0]
-    decls += prefixed(final.declare(spec.final_norm, spec.hidden_size), stem)
+    decls += _final_norm_decls(spec, final)
     # A tied checkpoint may still store the output projection; the stored tensor wins.
     decls.append(ParamDecl(spec.head_name, (spec.vocab_size, spec.hidden_size), "matrix", optional=True))
     for _, cls in _transforms(spec):
@@ -59,7 +75,7 @@ class LayerContext:
     the pages of the layer it reads from) and its state slots."""
 
     __slots__ = ("batch", "cache", "layer", "cache_layer", "writes_cache", "residual", "trace", "hand", "handed",
-                 "norm_after", "handed_out")
+                 "norm_after", "handed_out", "stream_rows")
 
     def __init__(self, batch, cache, layer: int, cache_layer: int, writes_cache: bool):
         self.batch = batch
@@ -79,6 +95,9 @@ class LayerContext:
         self.handed = None
         self.norm_after = None
         self.handed_out = None
+        # The rows of the stream in the model's type, where the part that last updated the stream left them
+        # (a block that normalises sublayer outputs does; any block may read, replace or clear them).
+        self.stream_rows = None
 
     def kv(self):
         return self.cache.layer_view(self.cache_layer, self.batch)
@@ -105,9 +124,8 @@ class DecoderModel:
             cls = lookup(BLOCKS, layer.block, "block")
             self.blocks.append(cls(layer, spec.hidden_size, scoped(params, layer.weight_prefix), dtype,
                                    self.device, self.shared))
-        stem = spec.final_norm_name.rsplit(".", 1)[0]
-        self.norm = lookup(NORMS, spec.final_norm.kind, "norm")(
-            spec.final_norm, spec.hidden_size, scoped(params, stem), dtype, self.device)
+        final = lookup(NORMS, spec.final_norm.kind, "norm")
+        self.norm = final(spec.final_norm, spec.hidden_size, _final_norm_params(spec, final, params), dtype, self.device)
         if spec.head_name in params:
             head = params[spec.head_name]
         elif spec.tie_word_embeddings:
@@ -172,6 +190,7 @@ class DecoderModel:
             top.record(self.spec.embed_name.rsplit(".", 1)[0] + ".out", resid)
         delta = None
         handed = None
+        stream_rows = None
         schedule = self.spec.schedule
         for at, entry in enumerate(schedule):
             own = entry.cache_from is None
@@ -179,10 +198,12 @@ class DecoderModel:
             if top is not None:
                 ctx.trace = top.child(self.spec.layers[entry.layer].weight_prefix)
             ctx.handed = handed
+            ctx.stream_rows = stream_rows
             if at + 1 < len(schedule):
                 ctx.norm_after = getattr(self.blocks[schedule[at + 1].layer], "first_norm", None)
             delta = self.blocks[entry.layer].forward(resid, delta, ctx)
             handed = ctx.handed_out if delta is None else None
+            stream_rows = ctx.stream_rows if delta is None else None
             if top is not None:
                 after = resid.clone()
                 if delta is not None:

@@ -60,6 +60,13 @@ class RmsNorm:
             return None
         return kernels.HandedNorm(self.gain32, self.eps, rows, self.width, device)
 
+    def apply_onto(self, resid: torch.Tensor, y: torch.Tensor, rows_dtype=None):
+        """resid += norm(y), for a layer that normalises a sublayer's output; ``y`` is 32-bit.  With
+        ``rows_dtype`` the updated rows of the stream come back in that type too, otherwise None."""
+        if not hasattr(self, "_gain32"):
+            self._gain32 = self.gain if self.gain.dtype == torch.float32 else self.gain.float()
+        return kernels.rmsnorm_onto(resid, y, self._gain32, self.eps, rows_dtype)
+
     def apply(self, resid: torch.Tensor, delta, out_dtype: torch.dtype, rows=None) -> torch.Tensor:
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.width), dtype=out_dtype, device=resid.device)
