@@ -1,6 +1,7 @@
 // The C interface of the host runtime.  Every call returns 0 (or a count) on
 // success and a negative number on failure; the message is read with
 // plh_last_error().  Handles are opaque pointers.
+#include <climits>
 #include <algorithm>
 #include <cstring>
 #include <string>
@@ -84,7 +85,11 @@ long plh_cache_tokens(void* c, uint64_t id) {
     return guarded([&] { return static_cast<long>(static_cast<CacheManager*>(c)->tokens(id)); });
 }
 long plh_cache_capacity(void* c, uint64_t id) {
-    return guarded([&] { return static_cast<long>(static_cast<CacheManager*>(c)->capacity(id)); });
+    // (a model none of whose layers keeps pages has room without end: the largest count, not a wrapped one)
+    return guarded([&] {
+        const size_t room = static_cast<CacheManager*>(c)->capacity(id);
+        return room > static_cast<size_t>(LONG_MAX) ? LONG_MAX : static_cast<long>(room);
+    });
 }
 long plh_cache_blocks_needed(void* c, uint64_t id, size_t count) {
     return guarded([&] { return static_cast<long>(static_cast<CacheManager*>(c)->blocks_needed(id, count)); });
@@ -165,6 +170,7 @@ long plh_cache_wasted_tokens(void* c, uint64_t id) {
     return guarded([&] { return static_cast<long>(static_cast<CacheManager*>(c)->wasted_tokens(id)); });
 }
 uint64_t plh_cache_counter(void* c, size_t group, int which) {
+    if (group >= static_cast<CacheManager*>(c)->num_groups()) return 0;     // (a model without pages has no pool to count)
     return pool_counter(static_cast<CacheManager*>(c)->pool(group), which);
 }
 long plh_cache_live_sequences(void* c) { return static_cast<long>(static_cast<CacheManager*>(c)->live_sequences()); }

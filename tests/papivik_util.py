@@ -1,0 +1,110 @@
+"""Configurations, model folders and comparisons for the tests of the Papivik design."""
+
+from __future__ import annotations
+
+import copy
+import json
+from pathlib import Path
+
+import torch
+
+import plain_papivik as plain
+
+
+def lightning(heads, dim, vdim, decay, mlp=None):
+    return {"type": "lightning", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "decay": list(decay)}, "mlp": mlp}
+
+
+def mlstm(heads, dim, vdim, cap, mlp=None):
+    return {"type": "mlstm", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "gate_cap": cap}, "mlp": mlp}
+
+
+def attention(heads, kv_heads, dim, vdim, conv, scale, rot=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv, "scale": scale}
+    if rot is not None:
+        m["rot"] = {"dims": rot[0], "base": rot[1]}
+    return m
+
+
+def delta(heads, kv_heads, dim, vdim, conv):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}
+
+
+def parallel(left, right, left_scale, right_scale, mlp=None):
+    return {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": left_scale, "right_scale": right_scale},
+            "mlp": mlp}
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def model(width, vocab, layers, eps=1e-6, scale=1.0):
+    return {"architecture": "Papivik", "embedding": {"scale": scale}, "layers": layers, "norm": {"eps": eps},
+            "vocab": vocab, "width": width}
+
+
+# Odd sizes: heads of 24 and 40 (no multiple of 16; value heads larger than key heads), a value head of 80 (two
+# column tiles of the scan), three query heads a key head, a rotation over a quarter of a head, two and three taps,
+# a feed-forward on some layers only, a vocabulary that is a prime.
+ODD = model(72, 211, [
+    mlstm(3, 24, 40, 8.0, dense(100)),
+    parallel(attention(6, 2, 24, 40, 2, 0.3, (8, 1000.0)), delta(4, 2, 16, 80, 3), 1.3, 0.7),
+    lightning(2, 80, 16, (0.9, 0.99), dense(64)),
+    parallel(attention(2, 2, 32, 16, 1, 0.2), delta(2, 2, 40, 24, 1), 0.5, 1.0, dense(96)),
+], eps=1e-5, scale=1.7)
+
+# What a small model tends to make equal or 1 is different here: one head, one key head for four query heads, a rotation
+# over the whole head, five taps, a scale of one, a width that is no multiple of eight.
+ONES = model(100, 97, [
+    parallel(attention(4, 1, 16, 16, 5, 1.0, (16, 50.0)), delta(1, 1, 48, 48, 2), 1.0, 1.0),
+    lightning(1, 16, 96, (0.5,)),
+    mlstm(1, 64, 16, 30.0),
+], eps=1e-6, scale=1.0)
+
+# Larger heads: rows of S beyond 64 and 128 (the scan's deepest shapes), value heads of 128, attention heads of 128.
+LARGE = model(256, 300, [
+    lightning(2, 128, 128, (0.97, 0.999)),
+    mlstm(2, 192, 96, 12.0),
+    parallel(attention(4, 2, 128, 128, 3, 0.09, (64, 10000.0)), delta(2, 1, 160, 64, 4), 0.8, 0.6, dense(320)),
+], eps=1e-6, scale=0.3)
+
+CONFIGS = {"odd": ODD, "ones": ONES, "large": LARGE}
+
+
+def write_model(folder, config, seed=0, dtype="float32", std=0.08, gain_std=0.2, edit=None) -> Path:
+    """A model folder with random weights from the package's random-weights mode; ``edit(tensors)`` may change
+    them (the folder is then written again)."""
+    from paged_llm_rs_amd.weights import write_random_model
+
+    folder = write_random_model(Path(folder), copy.deepcopy(config), seed=seed, std=std, gain_std=gain_std, dtype=dtype)
+    if edit is not None:
+        from safetensors.torch import load_file, save_file
+
+        tensors = load_file(str(folder / "model.safetensors"))
+        edit(tensors)
+        save_file({k: v.contiguous() for k, v in tensors.items()}, str(folder / "model.safetensors"))
+    return folder
+
+
+def load_plain(folder):
+    from safetensors.torch import load_file
+
+    config = json.loads((Path(folder) / "config.json").read_text())
+    weights = {k: v.to(torch.float64) for k, v in load_file(str(Path(folder) / "model.safetensors")).items()}
+    return config, weights
+
+
+def plain_logits(folder, prompts: dict) -> dict:
+    config, weights = load_plain(folder)
+    return {name: plain.forward(config, weights, tokens) for name, tokens in prompts.items()}
+
+
+def plain_greedy(folder, prompt, count: int) -> list:
+    config, weights = load_plain(folder)
+    tokens, out = list(prompt), []
+    for _ in range(count):
+        nxt = int(plain.forward(config, weights, tokens)[-1].argmax())
+        out.append(nxt)
+        tokens.append(nxt)
+    return out
