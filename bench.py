@@ -98,11 +98,12 @@ class DecodeBench:
         self.run_step, self.commit_step, self.kernels = run_step, commit_step, kernels
         self.runner = runner
         firsts = []
+        self.slots = {}
         for i in self.ids:
-            cache.manager.add_sequence(i)
+            self.slots[i] = cache.manager.add_sequence(i)       # (-1 for a model that keeps no state of its own)
             prompt = [rng.randrange(vocab) for _ in range(context)]
             assert cache.manager.reserve(i, context)
-            entry = [StepEntry(i, prompt, 0, [context - 1])]
+            entry = [StepEntry(i, prompt, 0, [context - 1], state_slot=self.slots[i], fresh_state=self.slots[i] >= 0)]
             logits = run_step(model, cache, entry)
             commit_step(cache, entry)
             firsts.append(int(kernels.argmax(logits).item()))
@@ -117,7 +118,8 @@ class DecodeBench:
             assert manager.reserve(i, 1)
         out = None
         if self.ahead and self.flight is not None:
-            entries = [self.StepEntry(i, [0], manager.tokens(i), [0], fed_row=row) for row, i in enumerate(self.ids)]
+            entries = [self.StepEntry(i, [0], manager.tokens(i), [0], state_slot=self.slots[i], fed_row=row)
+                       for row, i in enumerate(self.ids)]
             try:
                 out = self.runner.run(entries)
             except self.CannotFeed:
@@ -126,7 +128,8 @@ class DecodeBench:
             self.tokens = self.flight.greedy_on_host()
             self.flight = None
         if out is None:
-            entries = [self.StepEntry(i, [tok], manager.tokens(i), [0]) for i, tok in zip(self.ids, self.tokens)]
+            entries = [self.StepEntry(i, [tok], manager.tokens(i), [0], state_slot=self.slots[i])
+                       for i, tok in zip(self.ids, self.tokens)]
             out = self.runner.run(entries)
         self.commit_step(self.cache, entries)      # queued: written, for every step behind it
         self.flight = out
@@ -272,6 +275,87 @@ class Workbench:
         }
 
 
+# --only papivik: the Papivik design (layers of linear attention with fixed decays, of a matrix memory with
+# exponential gates, and of softmax attention with short convolutions beside a gated delta rule, each with a dense
+# feed-forward) at layer sizes of the Qwen3 shapes, beside Qwen3 dense with the same width, feed-forward width, layers
+# and vocabulary.  (name, width, feed-forward, heads of the attention, the Qwen3 shape beside it, layers)
+PAPIVIK_SIZES = {
+    "1k": (1024, 3072, 16, "0.6b", 6),
+    "4k": (4096, 12288, 32, "8b", 3),
+}
+
+
+def papivik_config(width: int, ff: int, heads: int, layers: int, vocab: int) -> dict:
+    mlp = {"kind": "dense", "ff": ff}
+    kinds = [
+        {"type": "lightning", "mixer": {"heads": heads // 2, "dim": 128, "vdim": 128,
+                                        "decay": [1.0 - 2.0 ** (-5 - 3 * h / max(heads // 2 - 1, 1)) for h in range(heads // 2)]}, "mlp": mlp},
+        {"type": "mlstm", "mixer": {"heads": heads // 4, "dim": 128, "vdim": 256, "gate_cap": 15.0}, "mlp": mlp},
+        {"type": "parallel", "mixer": {
+            "left": {"heads": heads, "kv_heads": 8, "dim": 128, "vdim": 128, "conv": 4, "scale": 128 ** -0.5,
+                     "rot": {"dims": 64, "base": 1000000.0}},
+            "right": {"heads": heads // 2, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "conv": 4},
+            "left_scale": 0.5, "right_scale": 0.5}, "mlp": mlp},
+    ]
+    return {"architecture": "Papivik", "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "vocab": vocab, "width": width,
+            "layers": [kinds[i % 3] for i in range(layers)]}
+
+
+def papivik_table(torch, args) -> int:
+    """Prefill of 2,048 tokens and decode at batch 8 and 64 from 512-token contexts, for the Papivik design and for
+    Qwen3 dense at the same width, layers and vocabulary; one JSON line."""
+    from paged_llm_rs_amd import write_random_model
+    from paged_llm_rs_amd.cache import PagedCache
+    from paged_llm_rs_amd.engine.batch import StepEntry
+    from paged_llm_rs_amd.engine.step import StepRunner, require_gpu
+    from paged_llm_rs_amd.parts.model import load_model
+
+    device = require_gpu("cuda:0")
+    context, out = 512, {}
+    for size, (width, ff, heads, beside, layers) in PAPIVIK_SIZES.items():
+        if args.size and size != args.size:
+            continue
+        vocab = COMMON["vocab_size"]
+        qwen = dict(SHAPES[beside][1], num_hidden_layers=layers, tie_word_embeddings=False)
+        for name, config in (("papivik", papivik_config(width, ff, heads, layers, vocab)), ("qwen3", qwen)):
+            with tempfile.TemporaryDirectory() as tmp:
+                say(f"{size}: writing and loading a random {layers}-layer {name} model of width {width}")
+                folder = write_random_model(Path(tmp) / "model", config, seed=0, std=0.02, gain_std=0.1, dtype="bfloat16")
+                _, model = load_model(folder, "bfloat16", device)
+            pages = (64 * (context + 2 * (args.steps + args.warmup) + 64) + 3 * PREFILL_TOKENS) // BLOCK_SIZE + 80
+            cache = PagedCache(model.cache_layout, BLOCK_SIZE, pages, torch.bfloat16, device, max_seqs=66)
+            runner = StepRunner(model, cache, graphs=not args.no_graphs)
+            point = {}
+            rng = random.Random(7)
+            for tokens in (PREFILL_TOKENS, 512):
+                prompt = [rng.randrange(vocab) for _ in range(tokens)]
+
+                def prefill():
+                    slot = cache.manager.add_sequence(1000)
+                    assert cache.manager.reserve(1000, tokens)
+                    runner.run([StepEntry(1000, prompt, 0, [tokens - 1], state_slot=slot, fresh_state=slot >= 0)])
+                    cache.manager.free_sequence(1000)
+
+                seconds = timed(prefill, 10, 4)
+                point[f"prefill_{tokens}_ms"] = round(seconds * 1e3, 3)
+                point[f"prefill_{tokens}_tokens_per_s"] = round(tokens / seconds, 1)
+            for batch in (8, 64):
+                bench = DecodeBench(model, cache, runner, batch, context, seed=batch)
+                seconds = timed(bench.step, args.steps, args.warmup)
+                bench.free()
+                point[f"decode_b{batch}_ms"] = round(seconds * 1e3, 3)
+                point[f"decode_b{batch}_tokens_per_s"] = round(batch / seconds, 1)
+            out[f"{size}_{name}"] = point
+            say(f"{size} {name}: {point}")
+            del runner, cache, model
+            import gc
+            gc.collect()
+            torch.cuda.empty_cache()
+    print(json.dumps({"papivik_beside_qwen3": out, "layers": {k: v[4] for k, v in PAPIVIK_SIZES.items()},
+                      "context": context, "dtype": "bf16", "data": "synthetic"}), flush=True)
+    return 0
+
+
 def products_table(torch) -> int:
     """Microseconds of y = x . w^T over large weight matrices that come from memory (several copies of each
     matrix in turn, inside one captured graph), by the library, the skinny and the streamed product, and
@@ -344,7 +428,8 @@ def main() -> int:
     parser.add_argument("--ahead", choices=["on", "off"], default="on",
                         help="--only engine: whether the engine queues a decoding step before it has read the tokens "
                              "of the one before")
-    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products"], default=None,
+    parser.add_argument("--size", choices=sorted(PAPIVIK_SIZES), default=None, help="--only papivik: one of its sizes alone")
+    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products", "papivik"], default=None,
                         help="run one part alone: the decode steps at --batch, the prefill, or (not part of the "
                              "default line) the whole engine on 1/4/16/32/64/128 requests at once, 16 prompt tokens and "
                              "128 generated each, as the reference's own table of clients does; mixed: one step of a "
@@ -352,7 +437,9 @@ def main() -> int:
                              "tables, first tokens behind a shared preamble with the prefix cache off and on, and the "
                              "gaps between the tokens of four running requests when a long prompt arrives, by --chunk; "
                              "products: the layer products of the 8B and 32B shapes at 8 to 64 rows, weights from memory, "
-                             "by the library and by the two hand-written products of few rows")
+                             "by the library and by the two hand-written products of few rows; papivik: prefill and decode "
+                             "of the Papivik design at layer sizes of the 0.6B and 8B shapes beside Qwen3 dense of the same "
+                             "width, layers and vocabulary")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")
@@ -362,6 +449,8 @@ def main() -> int:
 
     if args.only == "products":
         return products_table(torch)
+    if args.only == "papivik":
+        return papivik_table(torch, args)
 
     from paged_llm_rs_amd.engine.batch import StepEntry
     from paged_llm_rs_amd.engine.step import commit_step, require_gpu, run_step

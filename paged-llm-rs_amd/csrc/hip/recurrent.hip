@@ -6,11 +6,7 @@
 //
 // A request's tokens of the step are rows q_start[s] .. q_start[s] + q_len[s] - 1; its state lives in
 // slot state_slots[s] of a [slots, floats a slot] tensor.  A request without a slot (padding) is skipped.
-#include "common.hpp"
-
-#define PL_SCAN_LIGHTNING 0
-#define PL_SCAN_MLSTM 1
-#define PL_SCAN_DELTA 2
+#include "recurrent.hpp"
 
 #define PL_SCAN_CHUNK 16      // tokens staged in LDS at a time
 
@@ -19,29 +15,6 @@
     _Pragma("unroll") for (int ib = 0; ib < DMAX; ib += 16) \
         if (ib < D)                                   \
             _Pragma("unroll") for (int i = ib; i < ib + 16; ++i)
-
-struct ScanArgs {
-    const float* qkv;         // rows holding q, k and v (for the delta rule: already convolved and activated)
-    int qkv_stride, q_off, k_off, v_off;
-    const float* gates;       // rows holding the two pre-activations of the gates (mlstm: i, f; delta: beta, a)
-    int gates_stride, g1_off, g2_off;
-    const float* p1;          // lightning: decay a head; mlstm: bias of i; delta: A_log
-    const float* p2;          // mlstm: bias of f; delta: dt_bias
-    float cap;                // mlstm: the cap of the gates' pre-activations
-    float* state;             // [slots, state_stride]
-    long state_stride;
-    int s_off, n_off, m_off;  // where S [H, D, V], n [H, D] and m [H] start inside a slot
-    float* out;               // [rows, H * V]
-    const int* q_start;
-    const int* q_len;
-    const int* state_slots;
-    int H, G, D, V;           // heads, heads of q and k (G divides H), size of q and k, size of v
-};
-
-__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
-__device__ __forceinline__ float logsigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
-__device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + expf(-x)); }
-__device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); }
 
 // One wave owns 64 columns of one head's S for one request and walks the request's tokens in order.
 // Lane j holds column j of S (D values in registers), so S^T k and S^T q are sums inside a lane, taken
@@ -53,7 +26,7 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
     const int h = blockIdx.y, s = blockIdx.z;
     const int slot = a.state_slots[s];
     const int n = a.q_len[s];
-    if (slot < 0 || n <= 0) return;
+    if (slot < 0 || n <= 0 || (a.below > 0 && n >= a.below)) return;
     const int start = a.q_start[s];
     const int D = a.D, V = a.V, H = a.H;
     const int g = h / (H / a.G);
@@ -81,11 +54,14 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
     constexpr int NPER = (DMAX + 63) / 64;
     float nv[NPER];
     float m = 0.f;
+    // (Every tile of columns has a copy of n and m of its own in the slot, n [H, tiles, D] and m [H, tiles]: a
+    // tile that starts after another has finished must not read what that one wrote.)
+    const int tiles = gridDim.x;
     if (KIND == PL_SCAN_MLSTM) {
-        const float* ng = slot_state + a.n_off + static_cast<size_t>(h) * D;
+        const float* ng = slot_state + a.n_off + (static_cast<size_t>(h) * tiles + blockIdx.x) * D;
 #pragma unroll
         for (int r = 0; r < NPER; ++r) nv[r] = (lane + 64 * r < D) ? ng[lane + 64 * r] : 0.f;
-        m = slot_state[a.m_off + h];
+        m = slot_state[a.m_off + h * tiles + blockIdx.x];
     }
     float decay = 0.f, a_rate = 0.f, dt_bias = 0.f, bias_i = 0.f, bias_f = 0.f;
     if (KIND == PL_SCAN_LIGHTNING) decay = a.p1[h];
@@ -197,12 +173,12 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
         for (int i = 0; i < DMAX; ++i)
             if (i < D) Sg[static_cast<size_t>(i) * V + j] = S[i];
     }
-    if (KIND == PL_SCAN_MLSTM && blockIdx.x == 0) {
-        float* ng = slot_state + a.n_off + static_cast<size_t>(h) * D;
+    if (KIND == PL_SCAN_MLSTM) {
+        float* ng = slot_state + a.n_off + (static_cast<size_t>(h) * tiles + blockIdx.x) * D;
 #pragma unroll
         for (int r = 0; r < NPER; ++r)
             if (lane + 64 * r < D) ng[lane + 64 * r] = nv[r];
-        if (lane == 0) slot_state[a.m_off + h] = m;
+        if (lane == 0) slot_state[a.m_off + h * tiles + blockIdx.x] = m;
     }
 }
 
@@ -224,7 +200,7 @@ extern "C" int pl_recurrent_scan(int kind, const float* qkv, int qkv_stride, int
                                  const float* p1, const float* p2, float cap,
                                  float* state, long state_stride, int s_off, int n_off, int m_off,
                                  float* out, const int* q_start, const int* q_len, const int* state_slots,
-                                 int seqs, int H, int G, int D, int V, hipStream_t stream) {
+                                 int seqs, int H, int G, int D, int V, int below, hipStream_t stream) {
     PL_REQUIRE(kind >= 0 && kind <= 2, "recurrent_scan: kind %d", kind);
     PL_REQUIRE(H > 0 && G > 0 && H % G == 0, "recurrent_scan: %d heads over %d heads of q and k", H, G);
     PL_REQUIRE(D > 0 && D <= 256 && V > 0, "recurrent_scan: a state of %d by %d a head (q and k up to 256)", D, V);
@@ -235,7 +211,7 @@ extern "C" int pl_recurrent_scan(int kind, const float* qkv, int qkv_stride, int
     PL_REQUIRE(kind != PL_SCAN_MLSTM || cap > 0.f, "recurrent_scan: a gate cap of %g", cap);
     if (seqs == 0) return 0;
     ScanArgs a{qkv, qkv_stride, q_off, k_off, v_off, gates, gates_stride, g1_off, g2_off, p1, p2, cap,
-               state, state_stride, s_off, n_off, m_off, out, q_start, q_len, state_slots, H, G, D, V};
+               state, state_stride, s_off, n_off, m_off, out, q_start, q_len, state_slots, H, G, D, V, below};
     if (kind == PL_SCAN_LIGHTNING) return launch_scan<PL_SCAN_LIGHTNING>(a, seqs, stream);
     if (kind == PL_SCAN_MLSTM) return launch_scan<PL_SCAN_MLSTM>(a, seqs, stream);
     return launch_scan<PL_SCAN_DELTA>(a, seqs, stream);

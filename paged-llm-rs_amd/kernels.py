@@ -54,7 +54,10 @@ def _signatures(lib) -> None:
         "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, i, p],
         "pl_paged_attention_grouped_applies": [i, i, i, i],
         "pl_recurrent_scan": [i, p, i, i, i, i, p, i, i, i, p, p, f, p, ctypes.c_long, i, i, i, p, p, p, p,
-                              i, i, i, i, i, p],
+                              i, i, i, i, i, i, p],
+        "pl_recurrent_chunked": [i, p, i, i, i, i, p, i, i, i, p, p, f, p, ctypes.c_long, i, i, i, p, p, p, p,
+                                 i, i, i, i, i, i, p, p, p, p, p, p],
+        "pl_recurrent_chunk_tokens": [i],
         "pl_short_conv": [p, i, i, i, p, i, p, ctypes.c_long, i, p, p, p, p, p, i, i, p],
         "pl_conv_history": [p, i, i, i, i, p, ctypes.c_long, i, p, p, p, i, p],
         "pl_gated_group_norm": [p, i, i, i, p, i, f, p, i, i, i, p, i, p],
@@ -1045,6 +1048,9 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype,
 
 SCAN_KINDS = {"lightning": 0, "mlstm": 1, "delta": 2}
 SCAN_MAX_DIM = 256
+# A request that brings at least this many tokens to a step goes through the chunked kernels, where its mixer has
+# them (64 tokens at once instead of one after the other); the others, single tokens among them, go token by token.
+SCAN_CHUNKED_FROM = 16
 
 
 def _state_view(state: torch.Tensor, what: str):
@@ -1062,20 +1068,30 @@ def _step_rows(batch, n: int):
         _need(t, what, (count,), torch.int32)
 
 
+def scan_state_floats(kind: str, heads: int, dim: int, vdim: int) -> int:
+    """32-bit floats a request's state takes: the matrices S [heads, dim, vdim]; for ``mlstm`` also the normaliser n
+    and the running maximum m, a copy of each for every tile of 64 columns of vdim (the waves of a head's tiles
+    run on their own and keep equal copies): n [heads, tiles, dim], m [heads, tiles]."""
+    tiles = (vdim + 63) // 64
+    return heads * dim * vdim + (heads * tiles * (dim + 1) if kind == "mlstm" else 0)
+
+
 def recurrent_scan(kind: str, qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, state: torch.Tensor,
                    batch, heads: int, qk_heads: int, dim: int, vdim: int, *, gates: torch.Tensor | None = None,
                    g1_off: int = 0, g2_off: int = 0, p1: torch.Tensor | None = None, p2: torch.Tensor | None = None,
-                   cap: float = 0.0, out: torch.Tensor | None = None) -> torch.Tensor:
+                   cap: float = 0.0, out: torch.Tensor | None = None, chunked: bool = False) -> torch.Tensor:
     """The read-out [rows, heads * vdim] (32-bit) of a mixer that carries a [dim, vdim] matrix a head from
     token to token, over the tokens of a step, request by request, from and into the requests' state slots.
 
     ``lightning``: S = decay S + silu(k) silu(v)^T, o = S^T silu(q); ``p1`` = the decays.
     ``mlstm``: log gates i = cap tanh((x1 + b_i)/cap), f = logsigmoid(cap tanh((x2 + b_f)/cap)) from the two
     gate columns a head, a running maximum m, S and a normaliser n; ``p1``, ``p2`` = the biases; the state a
-    slot is S [heads, dim, vdim], n [heads, dim], m [heads].
+    slot is laid out as ``scan_state_floats`` says.
     ``delta``: ``qkv`` holds convolved and activated rows; q and k become unit vectors, beta = sigmoid(x1),
     decay = exp(-exp(A_log) softplus(x2 + dt_bias)); ``p1`` = A_log, ``p2`` = dt_bias.
-    q and k have ``qk_heads`` heads (head h of v reads head h / (heads / qk_heads))."""
+    q and k have ``qk_heads`` heads (head h of v reads head h / (heads / qk_heads)).
+    ``chunked`` (lightning with decays above zero, mlstm): requests that bring ``SCAN_CHUNKED_FROM`` tokens or more
+    are computed in chunks of tokens, the same sums in another order."""
     if kind not in SCAN_KINDS:
         raise TensorError(f"a scan of kind {kind!r}, the kernels know {', '.join(SCAN_KINDS)}")
     n = qkv.shape[0]
@@ -1089,7 +1105,8 @@ def recurrent_scan(kind: str, qkv: torch.Tensor, q_off: int, k_off: int, v_off: 
     if heads < 1 or qk_heads < 1 or heads % qk_heads or not 1 <= dim <= SCAN_MAX_DIM or vdim < 1:
         raise TensorError(f"a scan over {heads} heads ({qk_heads} of q and k) of {dim} by {vdim}")
     state, stride = _state_view(state, "the state")
-    need = heads * dim * vdim + (heads * dim + heads if kind == "mlstm" else 0)
+    tiles = (vdim + 63) // 64
+    need = scan_state_floats(kind, heads, dim, vdim)
     if state.shape[1] != need:
         raise TensorError(f"a state of {state.shape[1]} floats a slot, this mixer keeps {need}")
     _step_rows(batch, n)
@@ -1104,11 +1121,22 @@ def recurrent_scan(kind: str, qkv: torch.Tensor, q_off: int, k_off: int, v_off: 
         out = torch.empty((n, heads * vdim), dtype=torch.float32, device=qkv.device)
     _need(out, "read-out", (n, heads * vdim), torch.float32)
     hdv = heads * dim * vdim
-    _check(library().pl_recurrent_scan(
-        SCAN_KINDS[kind], qkv.data_ptr(), width, q_off, k_off, v_off, _ptr(gates),
-        0 if gates is None else gates.shape[1], g1_off, g2_off, _ptr(p1), _ptr(p2), float(cap),
-        state.data_ptr(), stride, 0, hdv, hdv + heads * dim, out.data_ptr(), batch.q_start.data_ptr(),
-        batch.q_len.data_ptr(), batch.state_slots.data_ptr(), batch.num_seqs, heads, qk_heads, dim, vdim, _stream()))
+    chunked = bool(chunked) and kind in ("lightning", "mlstm") and batch.max_q_len >= SCAN_CHUNKED_FROM
+    common = (SCAN_KINDS[kind], qkv.data_ptr(), width, q_off, k_off, v_off, _ptr(gates),
+              0 if gates is None else gates.shape[1], g1_off, g2_off, _ptr(p1), _ptr(p2), float(cap),
+              state.data_ptr(), stride, 0, hdv, hdv + heads * tiles * dim, out.data_ptr(), batch.q_start.data_ptr(),
+              batch.q_len.data_ptr(), batch.state_slots.data_ptr(), batch.num_seqs)
+    _check(library().pl_recurrent_scan(*common, heads, qk_heads, dim, vdim, SCAN_CHUNKED_FROM if chunked else 0, _stream()))
+    if chunked:
+        chunks = n // library().pl_recurrent_chunk_tokens(dim) + batch.num_seqs + 1
+        f32 = dict(dtype=torch.float32, device=qkv.device)
+        sums, before = torch.empty((chunks, hdv), **f32), torch.empty((chunks, hdv), **f32)
+        k_sums, n_before = (torch.empty((chunks, heads * dim), **f32), torch.empty((chunks, heads * dim), **f32)) \
+            if kind == "mlstm" else (None, None)
+        scalars = torch.empty((chunks, heads * 4), **f32)
+        _check(library().pl_recurrent_chunked(*common, batch.max_q_len, heads, dim, vdim, SCAN_CHUNKED_FROM,
+                                              sums.data_ptr(), _ptr(k_sums), before.data_ptr(), _ptr(n_before),
+                                              scalars.data_ptr(), _stream()))
     return out
 
 

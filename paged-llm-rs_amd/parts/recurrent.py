@@ -63,6 +63,8 @@ class LightningAttention(_ScanMixer):
         self.o_proj = Linear(params["o"])
         self.gain = _f32(params["norm"])
         self.decay = torch.tensor([float(d) for d in spec.decay], dtype=torch.float32, device=device)
+        # (in chunks a decay enters through its logarithm)
+        self.chunked = min(float(d) for d in spec.decay) > 0.0
         self.dtype = dtype
 
     def state_spec(self):
@@ -72,7 +74,7 @@ class LightningAttention(_ScanMixer):
         c = self.columns
         rows = self.proj.forward(x, out_dtype=torch.float32)
         read = kernels.recurrent_scan("lightning", rows, c["q"], c["k"], c["v"], ctx.state(), ctx.batch,
-                                      self.H, self.H, self.D, self.V, p1=self.decay)
+                                      self.H, self.H, self.D, self.V, p1=self.decay, chunked=self.chunked)
         normed = kernels.gated_group_norm(read, self.H * self.V, self.gain, self.spec.eps, self.dtype,
                                           gate=rows, gate_off=c["g"], gate_act="sigmoid")
         return self.o_proj.forward(normed, out_dtype=torch.float32)
@@ -101,15 +103,15 @@ class Mlstm(_ScanMixer):
         self.dtype = dtype
 
     def state_spec(self):
-        # S [H, D, V], the normaliser n [H, D], the running maximum m [H]
-        return StateSpec((self.H * self.D * self.V + self.H * self.D + self.H,), torch.float32)
+        # S, the normaliser n and the running maximum m (``kernels.scan_state_floats``)
+        return StateSpec((kernels.scan_state_floats("mlstm", self.H, self.D, self.V),), torch.float32)
 
     def forward(self, x, ctx):
         c = self.columns
         rows = self.proj.forward(x, out_dtype=torch.float32)
         read = kernels.recurrent_scan("mlstm", rows, c["q"], c["k"], c["v"], ctx.state(), ctx.batch,
                                       self.H, self.H, self.D, self.V, gates=rows, g1_off=c["i"], g2_off=c["f"],
-                                      p1=self.bias_i, p2=self.bias_f, cap=self.spec.gate_cap)
+                                      p1=self.bias_i, p2=self.bias_f, cap=self.spec.gate_cap, chunked=True)
         normed = kernels.gated_group_norm(read, self.V, self.gain, self.spec.eps, self.dtype,
                                           gate=rows, gate_off=c["g"], gate_act="sigmoid")
         return self.o_proj.forward(normed, out_dtype=torch.float32)
