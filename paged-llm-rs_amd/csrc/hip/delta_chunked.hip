@@ -1,0 +1,311 @@
+// Prompt portions through the gated delta rule in chunks of tokens.  For one head, with decays g_t,
+// G_t = g_1 ... g_t inside a chunk, and S_0 the state before the chunk, the rule
+//     S_t = g_t S_(t-1) + k_t u_t^T ,   u_t = beta_t (v_t - g_t S_(t-1)^T k_t)
+// unrolls to  S_t = G_t S_0 + sum_{s<=t} (G_t / G_s) k_s u_s^T , and the u of a chunk solve
+//     (I + M) U = R ,  M[t][s] = beta_t (G_t / G_s) (k_t . k_s) for s < t ,  R_t = beta_t (v_t - G_t S_0^T k_t) .
+// `prepare` (every chunk and head at once) makes k and q unit vectors, and computes T = (I + M)^-1 by
+// forward substitution and Aq[t][s] = (G_t / G_s) (q_t . k_s) for s <= t.  `walk` (one workgroup for a
+// request, a head and 16 columns of the state) then goes through the chunks in order:
+//     R = beta (V - G K S) ;  U = T R ;  O = G Q S + Aq U ;  S = G_L S + (K weighted by G_L / G_s)^T U .
+// 32-bit throughout, on the vector units, sums in a fixed order.
+#include "recurrent.hpp"
+
+struct DeltaArgs {
+    ScanArgs a;
+    float* Kn;       // [chunks, H, C, D]  k as unit vectors
+    float* Qn;       // [chunks, H, C, D]  q as unit vectors times D^-1/2
+    float* Tm;       // [chunks, H, C, C]  (I + M)^-1
+    float* Aq;       // [chunks, H, C, C]
+    float* scal;     // [chunks, H, 3, C]  G_t; beta_t; G_L / G_t
+};
+
+template <int C>
+__device__ __forceinline__ int delta_chunk_number(const ScanArgs& a, int s, int c) { return a.q_start[s] / C + s + c; }
+
+template <int C>
+__global__ __launch_bounds__(256) void delta_prepare_kernel(DeltaArgs da) {
+    const ScanArgs& a = da.a;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int TT = C / 16;
+    const int D = a.D, H = a.H;
+    const int c = blockIdx.x, h = blockIdx.y, s = blockIdx.z;
+    const int slot = a.state_slots[s], n = a.q_len[s];
+    if (slot < 0 || n < a.below || c * C >= n) return;
+    const int L = min(C, n - c * C), row0 = a.q_start[s] + c * C;
+    const int g = h / (H / a.G);
+    const size_t idx = static_cast<size_t>(delta_chunk_number<C>(a, s, c)) * H + h;
+    const int Dq = ((D + 3) & ~3) + 4;
+    float* qs = lds;                 // [C][Dq]
+    float* ks = qs + C * Dq;         // [C][Dq]
+    float* M = ks + C * Dq;          // [C][C + 1]
+    float* bs = M + C * (C + 1);     // [C]
+    float* be = bs + C;              // [C]
+    float* nrm = be + C;             // [2 C]
+    const int tid = threadIdx.x;
+    for (int e = tid; e < C * Dq; e += 256) {
+        const int t = e / Dq, i = e - t * Dq;
+        float q = 0.f, k = 0.f;
+        if (t < L && i < D) {
+            const float* row = a.qkv + static_cast<size_t>(row0 + t) * a.qkv_stride;
+            q = row[a.q_off + g * D + i];
+            k = row[a.k_off + g * D + i];
+        }
+        qs[e] = q;
+        ks[e] = k;
+    }
+    if (tid == 0) {
+        const float rate = expf(a.p1[h]), dt_bias = a.p2[h];
+        float sum = 0.f;
+        for (int t = 0; t < C; ++t) {
+            float beta = 0.f;
+            if (t < L) {
+                const float* row = a.gates + static_cast<size_t>(row0 + t) * a.gates_stride;
+                beta = sigmoid_f(row[a.g1_off + h]);
+                sum += -rate * softplus_f(row[a.g2_off + h] + dt_bias);
+            }
+            bs[t] = sum;
+            be[t] = beta;
+        }
+    }
+    __syncthreads();
+    if (tid < 2 * C) {
+        const float* x = (tid < C ? qs : ks) + (tid < C ? tid : tid - C) * Dq;
+        float ss = 0.f;
+        for (int i = 0; i < D; ++i) ss += x[i] * x[i];
+        nrm[tid] = 1.f / sqrtf(ss + 1e-6f) * (tid < C ? 1.f / sqrtf(static_cast<float>(D)) : 1.f);
+    }
+    __syncthreads();
+    for (int e = tid; e < C * Dq; e += 256) {
+        const int t = e / Dq;
+        qs[e] *= nrm[t];
+        ks[e] *= nrm[C + t];
+    }
+    __syncthreads();
+    // the unit vectors and the chunk's scalars go out for the walk
+    float* Kn = da.Kn + idx * C * D;
+    float* Qn = da.Qn + idx * C * D;
+    for (int e = tid; e < C * D; e += 256) {
+        const int t = e / D, i = e - t * D;
+        Kn[e] = ks[t * Dq + i];
+        Qn[e] = qs[t * Dq + i];
+    }
+    float* scal = da.scal + idx * 3 * C;
+    if (tid < C) {
+        scal[tid] = expf(bs[tid]);
+        scal[C + tid] = be[tid];
+        scal[2 * C + tid] = tid < L ? expf(bs[L - 1] - bs[tid]) : 0.f;
+    }
+    const int ty = tid / 16, tx = tid % 16;
+    {
+        float kk[TT][TT], qk[TT][TT];
+#pragma unroll
+        for (int i = 0; i < TT; ++i)
+#pragma unroll
+            for (int j = 0; j < TT; ++j) kk[i][j] = qk[i][j] = 0.f;
+        for (int d = 0; d < Dq - 4; d += 4) {
+            float4 qv[TT], kt[TT], kv[TT];
+#pragma unroll
+            for (int i = 0; i < TT; ++i) {
+                qv[i] = *reinterpret_cast<const float4*>(qs + (ty + 16 * i) * Dq + d);
+                kt[i] = *reinterpret_cast<const float4*>(ks + (ty + 16 * i) * Dq + d);
+            }
+#pragma unroll
+            for (int j = 0; j < TT; ++j) kv[j] = *reinterpret_cast<const float4*>(ks + (tx + 16 * j) * Dq + d);
+#pragma unroll
+            for (int i = 0; i < TT; ++i)
+#pragma unroll
+                for (int j = 0; j < TT; ++j) {
+                    kk[i][j] += kt[i].x * kv[j].x + kt[i].y * kv[j].y + kt[i].z * kv[j].z + kt[i].w * kv[j].w;
+                    qk[i][j] += qv[i].x * kv[j].x + qv[i].y * kv[j].y + qv[i].z * kv[j].z + qv[i].w * kv[j].w;
+                }
+        }
+        float* Aq = da.Aq + idx * C * C;
+#pragma unroll
+        for (int i = 0; i < TT; ++i)
+#pragma unroll
+            for (int j = 0; j < TT; ++j) {
+                const int t = ty + 16 * i, u = tx + 16 * j;
+                const float w = (u <= t && t < L) ? expf(bs[t] - bs[u]) : 0.f;
+                M[t * (C + 1) + u] = u < t ? be[t] * w * kk[i][j] : 0.f;
+                Aq[t * C + u] = w * qk[i][j];
+            }
+    }
+    __syncthreads();
+    // T = (I + M)^-1, a column a thread: T[t][j] = [t == j] - sum_{s < t} M[t][s] T[s][j]
+    if (tid < C) {
+        float col[C];
+#pragma unroll
+        for (int t = 0; t < C; ++t) {
+            float val = t == tid ? 1.f : 0.f;
+#pragma unroll
+            for (int u = 0; u < t; ++u) val -= M[t * (C + 1) + u] * col[u];
+            col[t] = val;
+        }
+        float* Tm = da.Tm + idx * C * C;
+#pragma unroll
+        for (int t = 0; t < C; ++t) Tm[t * C + tid] = col[t];
+    }
+}
+
+// One workgroup: a request, a head, 16 columns of the state; the chunks in order.
+template <int C>
+__global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
+    const ScanArgs& a = da.a;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int D = a.D, V = a.V, H = a.H;
+    const int v0 = blockIdx.x * 16, h = blockIdx.y, s = blockIdx.z;
+    const int slot = a.state_slots[s], n = a.q_len[s];
+    if (slot < 0 || n < a.below) return;
+    const int chunks = (n + C - 1) / C;
+    const int Dq = ((D + 3) & ~3) + 4, Dr = (D + 3) & ~3;
+    float* qs = lds;                 // [C][Dq]
+    float* ks = qs + C * Dq;         // [C][Dq]
+    float* Tm = ks + C * Dq;         // [C][C + 1]
+    float* Aq = Tm + C * (C + 1);    // [C][C + 1]
+    float* S = Aq + C * (C + 1);     // [Dr][16]
+    float* Vt = S + Dr * 16;         // [C][16]
+    float* R = Vt + C * 16;          // [C][16]
+    float* U = R + C * 16;           // [C][16]
+    float* sc = U + C * 16;          // [3][C]
+    const int tid = threadIdx.x;
+    float* Sg = a.state + static_cast<size_t>(slot) * a.state_stride + a.s_off + static_cast<size_t>(h) * D * V;
+    for (int e = tid; e < Dr * 16; e += 256) {
+        const int d = e / 16, v = v0 + (e & 15);
+        S[e] = (d < D && v < V) ? Sg[static_cast<size_t>(d) * V + v] : 0.f;
+    }
+    const int first = delta_chunk_number<C>(a, s, 0);
+    // a thread's rows and columns in the products with C rows: row t, columns vq * 4 .. + 3 (C = 64), or two
+    // columns (C = 32: 32 rows by 8 pairs)
+    constexpr int PER = C == 64 ? 4 : 2;
+    const int t_row = tid / (16 / PER), vq = (tid % (16 / PER)) * PER;
+    for (int c = 0; c < chunks; ++c) {
+        const size_t idx = static_cast<size_t>(first + c) * H + h;
+        const int L = min(C, n - c * C), row0 = a.q_start[s] + c * C;
+        __syncthreads();
+        {
+            const float* Kn = da.Kn + idx * C * D;
+            const float* Qn = da.Qn + idx * C * D;
+            for (int e = tid; e < C * Dq; e += 256) {
+                const int t = e / Dq, i = e - t * Dq;
+                const bool in = i < D;
+                ks[e] = in ? Kn[t * D + i] : 0.f;
+                qs[e] = in ? Qn[t * D + i] : 0.f;
+            }
+            const float* Tg = da.Tm + idx * C * C;
+            const float* Ag = da.Aq + idx * C * C;
+            for (int e = tid; e < C * C; e += 256) {
+                const int t = e / C, u = e - t * C;
+                Tm[t * (C + 1) + u] = Tg[e];
+                Aq[t * (C + 1) + u] = Ag[e];
+            }
+            for (int e = tid; e < C * 16; e += 256) {
+                const int t = e / 16, v = v0 + (e & 15);
+                Vt[e] = (t < L && v < V) ? a.qkv[static_cast<size_t>(row0 + t) * a.qkv_stride + a.v_off + h * V + v] : 0.f;
+            }
+            for (int e = tid; e < 3 * C; e += 256) sc[e] = da.scal[idx * 3 * C + e];
+        }
+        __syncthreads();
+        // K S and Q S for the thread's row
+        float ksum[PER], qsum[PER];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) ksum[j] = qsum[j] = 0.f;
+        for (int d = 0; d < Dr; ++d) {
+            const float kd = ks[t_row * Dq + d], qd = qs[t_row * Dq + d];
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                const float sv = S[d * 16 + vq + j];
+                ksum[j] += kd * sv;
+                qsum[j] += qd * sv;
+            }
+        }
+        const float gam = sc[t_row], beta = sc[C + t_row];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) R[t_row * 16 + vq + j] = beta * (Vt[t_row * 16 + vq + j] - gam * ksum[j]);
+        __syncthreads();
+        float us[PER];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) us[j] = 0.f;
+        for (int u = 0; u <= t_row; ++u) {
+            const float w = Tm[t_row * (C + 1) + u];
+#pragma unroll
+            for (int j = 0; j < PER; ++j) us[j] += w * R[u * 16 + vq + j];
+        }
+#pragma unroll
+        for (int j = 0; j < PER; ++j) U[t_row * 16 + vq + j] = us[j];
+        __syncthreads();
+        float os[PER];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) os[j] = gam * qsum[j];
+        for (int u = 0; u <= t_row; ++u) {
+            const float w = Aq[t_row * (C + 1) + u];
+#pragma unroll
+            for (int j = 0; j < PER; ++j) os[j] += w * U[u * 16 + vq + j];
+        }
+        if (t_row < L) {
+#pragma unroll
+            for (int j = 0; j < PER; ++j)
+                if (v0 + vq + j < V)
+                    a.out[static_cast<size_t>(row0 + t_row) * (H * V) + h * V + v0 + vq + j] = os[j];
+        }
+        // S = G_L S + sum_s (G_L / G_s) k_s u_s^T : a thread owns a row d of S and 8 of its 16 columns
+        const float gl = sc[L - 1];
+        for (int d = tid / 2; d < Dr; d += 128) {
+            const int half = (tid & 1) * 8;
+            float acc[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = gl * S[d * 16 + half + j];
+            for (int u = 0; u < L; ++u) {
+                const float kw = ks[u * Dq + d] * sc[2 * C + u];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[j] += kw * U[u * 16 + half + j];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) S[d * 16 + half + j] = acc[j];
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < Dr * 16; e += 256) {
+        const int d = e / 16, v = v0 + (e & 15);
+        if (d < D && v < V) Sg[static_cast<size_t>(d) * V + v] = S[e];
+    }
+}
+
+template <int C>
+static int launch_delta(const DeltaArgs& da, int seqs, int max_q_len, hipStream_t stream) {
+    const ScanArgs& a = da.a;
+    const int Dq = ((a.D + 3) & ~3) + 4, Dr = (a.D + 3) & ~3;
+    const size_t lds_p = (2 * static_cast<size_t>(C) * Dq + C * (C + 1) + 4 * C) * sizeof(float);
+    const size_t lds_w = (2 * static_cast<size_t>(C) * Dq + 2 * C * (C + 1) + Dr * 16 + 3 * C * 16 + 3 * C) * sizeof(float);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&delta_prepare_kernel<C>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_p));
+    PL_REQUIRE(e == hipSuccess, "delta_chunked: %zu bytes of LDS refused: %s", lds_p, hipGetErrorString(e));
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&delta_walk_kernel<C>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_w));
+    PL_REQUIRE(e == hipSuccess, "delta_chunked: %zu bytes of LDS refused: %s", lds_w, hipGetErrorString(e));
+    delta_prepare_kernel<C><<<dim3(pl_ceil_div(max_q_len, C), a.H, seqs), 256, lds_p, stream>>>(da);
+    PL_CHECK_LAUNCH("delta_chunked (prepare)");
+    delta_walk_kernel<C><<<dim3(pl_ceil_div(a.V, 16), a.H, seqs), 256, lds_w, stream>>>(da);
+    PL_CHECK_LAUNCH("delta_chunked (walk)");
+    return 0;
+}
+
+// The requests of the step that bring at least `from` tokens.  Kn, Qn: room for (rows / chunk + requests)
+// chunks of H * chunk * D floats; Tm, Aq: of H * chunk * chunk; scal: of H * 3 * chunk.
+extern "C" int pl_delta_chunked(const float* qkv, int qkv_stride, int q_off, int k_off, int v_off,
+                                const float* gates, int gates_stride, int g1_off, int g2_off,
+                                const float* a_log, const float* dt_bias,
+                                float* state, long state_stride, float* out,
+                                const int* q_start, const int* q_len, const int* state_slots,
+                                int seqs, int max_q_len, int H, int G, int D, int V, int from,
+                                float* Kn, float* Qn, float* Tm, float* Aq, float* scal, hipStream_t stream) {
+    PL_REQUIRE(H > 0 && G > 0 && H % G == 0 && D > 0 && D <= 256 && V > 0 && from >= 1,
+               "delta_chunked: %d heads over %d of q and k, %d by %d, from %d tokens", H, G, D, V, from);
+    PL_REQUIRE(gates != nullptr && a_log != nullptr && dt_bias != nullptr, "delta_chunked: the gates are missing");
+    PL_REQUIRE(Kn != nullptr && Qn != nullptr && Tm != nullptr && Aq != nullptr && scal != nullptr, "delta_chunked: no room for the chunks");
+    PL_REQUIRE(seqs >= 0 && seqs <= 65535 && H <= 65535, "delta_chunked: %d requests, %d heads", seqs, H);
+    if (seqs == 0 || max_q_len < from) return 0;
+    DeltaArgs da{{qkv, qkv_stride, q_off, k_off, v_off, gates, gates_stride, g1_off, g2_off, a_log, dt_bias, 0.f, state,
+                  state_stride, 0, 0, 0, out, q_start, q_len, state_slots, H, G, D, V, from},
+                 Kn, Qn, Tm, Aq, scal};
+    return D <= 128 ? launch_delta<64>(da, seqs, max_q_len, stream) : launch_delta<32>(da, seqs, max_q_len, stream);
+}

@@ -58,6 +58,8 @@ def _signatures(lib) -> None:
         "pl_recurrent_chunked": [i, p, i, i, i, i, p, i, i, i, p, p, f, p, ctypes.c_long, i, i, i, p, p, p, p,
                                  i, i, i, i, i, i, p, p, p, p, p, p],
         "pl_recurrent_chunk_tokens": [i],
+        "pl_delta_chunked": [p, i, i, i, i, p, i, i, i, p, p, p, ctypes.c_long, p, p, p, p, i, i, i, i, i, i, i,
+                             p, p, p, p, p, p],
         "pl_short_conv": [p, i, i, i, p, i, p, ctypes.c_long, i, p, p, p, p, p, i, i, p],
         "pl_conv_history": [p, i, i, i, i, p, ctypes.c_long, i, p, p, p, i, p],
         "pl_gated_group_norm": [p, i, i, i, p, i, f, p, i, i, i, p, i, p],
@@ -1090,7 +1092,7 @@ def recurrent_scan(kind: str, qkv: torch.Tensor, q_off: int, k_off: int, v_off: 
     ``delta``: ``qkv`` holds convolved and activated rows; q and k become unit vectors, beta = sigmoid(x1),
     decay = exp(-exp(A_log) softplus(x2 + dt_bias)); ``p1`` = A_log, ``p2`` = dt_bias.
     q and k have ``qk_heads`` heads (head h of v reads head h / (heads / qk_heads)).
-    ``chunked`` (lightning with decays above zero, mlstm): requests that bring ``SCAN_CHUNKED_FROM`` tokens or more
+    ``chunked`` (lightning only with decays above zero): requests that bring ``SCAN_CHUNKED_FROM`` tokens or more
     are computed in chunks of tokens, the same sums in another order."""
     if kind not in SCAN_KINDS:
         raise TensorError(f"a scan of kind {kind!r}, the kernels know {', '.join(SCAN_KINDS)}")
@@ -1121,13 +1123,26 @@ def recurrent_scan(kind: str, qkv: torch.Tensor, q_off: int, k_off: int, v_off: 
         out = torch.empty((n, heads * vdim), dtype=torch.float32, device=qkv.device)
     _need(out, "read-out", (n, heads * vdim), torch.float32)
     hdv = heads * dim * vdim
-    chunked = bool(chunked) and kind in ("lightning", "mlstm") and batch.max_q_len >= SCAN_CHUNKED_FROM
+    chunked = bool(chunked) and batch.max_q_len >= SCAN_CHUNKED_FROM
     common = (SCAN_KINDS[kind], qkv.data_ptr(), width, q_off, k_off, v_off, _ptr(gates),
               0 if gates is None else gates.shape[1], g1_off, g2_off, _ptr(p1), _ptr(p2), float(cap),
               state.data_ptr(), stride, 0, hdv, hdv + heads * tiles * dim, out.data_ptr(), batch.q_start.data_ptr(),
               batch.q_len.data_ptr(), batch.state_slots.data_ptr(), batch.num_seqs)
     _check(library().pl_recurrent_scan(*common, heads, qk_heads, dim, vdim, SCAN_CHUNKED_FROM if chunked else 0, _stream()))
-    if chunked:
+    if chunked and kind == "delta":
+        tokens = library().pl_recurrent_chunk_tokens(dim)
+        chunks = (n // tokens + batch.num_seqs + 1) * heads
+        f32 = dict(dtype=torch.float32, device=qkv.device)
+        unit_k, unit_q = torch.empty((chunks, tokens * dim), **f32), torch.empty((chunks, tokens * dim), **f32)
+        inverse, masked = torch.empty((chunks, tokens * tokens), **f32), torch.empty((chunks, tokens * tokens), **f32)
+        scalars = torch.empty((chunks, 3 * tokens), **f32)
+        _check(library().pl_delta_chunked(
+            qkv.data_ptr(), width, q_off, k_off, v_off, gates.data_ptr(), gates.shape[1], g1_off, g2_off,
+            p1.data_ptr(), p2.data_ptr(), state.data_ptr(), stride, out.data_ptr(), batch.q_start.data_ptr(),
+            batch.q_len.data_ptr(), batch.state_slots.data_ptr(), batch.num_seqs, batch.max_q_len, heads, qk_heads, dim,
+            vdim, SCAN_CHUNKED_FROM, unit_k.data_ptr(), unit_q.data_ptr(), inverse.data_ptr(), masked.data_ptr(),
+            scalars.data_ptr(), _stream()))
+    elif chunked:
         chunks = n // library().pl_recurrent_chunk_tokens(dim) + batch.num_seqs + 1
         f32 = dict(dtype=torch.float32, device=qkv.device)
         sums, before = torch.empty((chunks, hdv), **f32), torch.empty((chunks, hdv), **f32)

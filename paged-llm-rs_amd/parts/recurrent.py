@@ -160,7 +160,7 @@ class GatedDelta(_ScanMixer):
         kernels.conv_history(rows, c["q"], self.conv_w, history, ctx.batch)
         read = kernels.recurrent_scan("delta", mixed, 0, G * D, 2 * G * D, state[:, :self.matrix], ctx.batch,
                                       self.H, G, D, self.V, gates=rows, g1_off=c["b"], g2_off=c["a"],
-                                      p1=self.a_log, p2=self.dt_bias)
+                                      p1=self.a_log, p2=self.dt_bias, chunked=True)
         normed = kernels.gated_group_norm(read, self.V, self.gain, self.spec.eps, self.dtype,
                                           gate=rows, gate_off=c["g"], gate_act="silu")
         return self.o_proj.forward(normed, out_dtype=torch.float32)
