@@ -12,12 +12,24 @@
 
 struct DeltaArgs {
     ScanArgs a;
-    float* Kn;       // [chunks, H, C, D]  k as unit vectors
-    float* Qn;       // [chunks, H, C, D]  q as unit vectors times D^-1/2
+    float* Kn;       // [chunks, H, C, Dr]  k as unit vectors, rows of Dr = D rounded up to 4
+    float* Qn;       // [chunks, H, C, Dr]  q as unit vectors times D^-1/2
     float* Tm;       // [chunks, H, C, C]  (I + M)^-1
     float* Aq;       // [chunks, H, C, C]
     float* scal;     // [chunks, H, 3, C]  G_t; beta_t; G_L / G_t
 };
+
+// PER (4 or 2) neighbouring values of a 16-column row in LDS, in one read (the rows start on 64 bytes).
+template <int PER>
+__device__ __forceinline__ void read_run(const float* p, float* out) {
+    if (PER == 4) {
+        const float4 x = *reinterpret_cast<const float4*>(p);
+        out[0] = x.x; out[1] = x.y; out[2] = x.z; out[3] = x.w;
+    } else {
+        const float2 x = *reinterpret_cast<const float2*>(p);
+        out[0] = x.x; out[1] = x.y;
+    }
+}
 
 template <int C>
 __device__ __forceinline__ int delta_chunk_number(const ScanArgs& a, int s, int c) { return a.q_start[s] / C + s + c; }
@@ -82,10 +94,11 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(DeltaArgs da) {
     }
     __syncthreads();
     // the unit vectors and the chunk's scalars go out for the walk
-    float* Kn = da.Kn + idx * C * D;
-    float* Qn = da.Qn + idx * C * D;
-    for (int e = tid; e < C * D; e += 256) {
-        const int t = e / D, i = e - t * D;
+    const int Dr = Dq - 4;          // (rows of whole quads, zeros behind D: the walk fetches them in quads)
+    float* Kn = da.Kn + idx * C * Dr;
+    float* Qn = da.Qn + idx * C * Dr;
+    for (int e = tid; e < C * Dr; e += 256) {
+        const int t = e / Dr, i = e - t * Dr;
         Kn[e] = ks[t * Dq + i];
         Qn[e] = qs[t * Dq + i];
     }
@@ -147,7 +160,9 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(DeltaArgs da) {
     }
 }
 
-// One workgroup: a request, a head, 16 columns of the state; the chunks in order.
+// One workgroup: a request, a head, 16 columns of the state; the chunks in order.  What a chunk needs
+// (its unit vectors, T, Aq, the columns of v, the scalars) is asked for while the chunk before is computed
+// and waits in registers: with one workgroup a compute unit nothing else would hide the trip to memory.
 template <int C>
 __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
     const ScanArgs& a = da.a;
@@ -157,7 +172,7 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
     const int slot = a.state_slots[s], n = a.q_len[s];
     if (slot < 0 || n < a.below) return;
     const int chunks = (n + C - 1) / C;
-    const int Dq = ((D + 3) & ~3) + 4, Dr = (D + 3) & ~3;
+    const int Dr = (D + 3) & ~3, Dq = Dr + 4;
     float* qs = lds;                 // [C][Dq]
     float* ks = qs + C * Dq;         // [C][Dq]
     float* Tm = ks + C * Dq;         // [C][C + 1]
@@ -174,48 +189,93 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
         S[e] = (d < D && v < V) ? Sg[static_cast<size_t>(d) * V + v] : 0.f;
     }
     const int first = delta_chunk_number<C>(a, s, 0);
-    // a thread's rows and columns in the products with C rows: row t, columns vq * 4 .. + 3 (C = 64), or two
-    // columns (C = 32: 32 rows by 8 pairs)
+    // a thread's row and columns in the products with C rows: row t, columns vq .. vq + PER - 1
     constexpr int PER = C == 64 ? 4 : 2;
     const int t_row = tid / (16 / PER), vq = (tid % (16 / PER)) * PER;
-    for (int c = 0; c < chunks; ++c) {
+    const int row_bound = (tid / 64 + 1) * (64 / (16 / PER));      // one past the last row of this thread's wave
+
+    // what a thread fetches of a chunk: up to KQ quads of k and of q, TA quads of T and of Aq, VS values of v
+    constexpr int KQ = 8, TA = C * C / 4 / 256 > 0 ? C * C / 4 / 256 : 1, VS = C * 16 / 256;
+    const int quads_row = Dr / 4, kq_quads = C * quads_row;
+    int kq_at[KQ];
+#pragma unroll
+    for (int r = 0; r < KQ; ++r) {
+        const int f = tid + 256 * r;
+        kq_at[r] = f < kq_quads ? (f / quads_row) * Dq + (f % quads_row) * 4 : -1;
+    }
+    float4 kreg[KQ], qreg[KQ], treg[TA], areg[TA];
+    float vreg[VS], sreg = 0.f;
+    auto fetch = [&](int c) {
         const size_t idx = static_cast<size_t>(first + c) * H + h;
+        const float4* Kn = reinterpret_cast<const float4*>(da.Kn + idx * C * Dr);
+        const float4* Qn = reinterpret_cast<const float4*>(da.Qn + idx * C * Dr);
+#pragma unroll
+        for (int r = 0; r < KQ; ++r)
+            if (kq_at[r] >= 0) {
+                kreg[r] = Kn[tid + 256 * r];
+                qreg[r] = Qn[tid + 256 * r];
+            }
+        const float4* Tg = reinterpret_cast<const float4*>(da.Tm + idx * C * C);
+        const float4* Ag = reinterpret_cast<const float4*>(da.Aq + idx * C * C);
+#pragma unroll
+        for (int r = 0; r < TA; ++r)
+            if (tid + 256 * r < C * C / 4) {
+                treg[r] = Tg[tid + 256 * r];
+                areg[r] = Ag[tid + 256 * r];
+            }
+        const int L = min(C, n - c * C), row0 = a.q_start[s] + c * C;
+#pragma unroll
+        for (int r = 0; r < VS; ++r) {
+            const int e = tid + 256 * r, t = e / 16, v = v0 + (e & 15);
+            vreg[r] = (t < L && v < V) ? a.qkv[static_cast<size_t>(row0 + t) * a.qkv_stride + a.v_off + h * V + v] : 0.f;
+        }
+        if (tid < 3 * C) sreg = da.scal[idx * 3 * C + tid];
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int r = 0; r < KQ; ++r)
+            if (kq_at[r] >= 0) {
+                *reinterpret_cast<float4*>(ks + kq_at[r]) = kreg[r];
+                *reinterpret_cast<float4*>(qs + kq_at[r]) = qreg[r];
+            }
+#pragma unroll
+        for (int r = 0; r < TA; ++r) {
+            const int f = tid + 256 * r;
+            if (f < C * C / 4) {
+                const int at = (f / (C / 4)) * (C + 1) + (f % (C / 4)) * 4;
+                Tm[at] = treg[r].x; Tm[at + 1] = treg[r].y; Tm[at + 2] = treg[r].z; Tm[at + 3] = treg[r].w;
+                Aq[at] = areg[r].x; Aq[at + 1] = areg[r].y; Aq[at + 2] = areg[r].z; Aq[at + 3] = areg[r].w;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < VS; ++r) Vt[tid + 256 * r] = vreg[r];
+        if (tid < 3 * C) sc[tid] = sreg;
+    };
+    fetch(0);
+    for (int c = 0; c < chunks; ++c) {
         const int L = min(C, n - c * C), row0 = a.q_start[s] + c * C;
         __syncthreads();
-        {
-            const float* Kn = da.Kn + idx * C * D;
-            const float* Qn = da.Qn + idx * C * D;
-            for (int e = tid; e < C * Dq; e += 256) {
-                const int t = e / Dq, i = e - t * Dq;
-                const bool in = i < D;
-                ks[e] = in ? Kn[t * D + i] : 0.f;
-                qs[e] = in ? Qn[t * D + i] : 0.f;
-            }
-            const float* Tg = da.Tm + idx * C * C;
-            const float* Ag = da.Aq + idx * C * C;
-            for (int e = tid; e < C * C; e += 256) {
-                const int t = e / C, u = e - t * C;
-                Tm[t * (C + 1) + u] = Tg[e];
-                Aq[t * (C + 1) + u] = Ag[e];
-            }
-            for (int e = tid; e < C * 16; e += 256) {
-                const int t = e / 16, v = v0 + (e & 15);
-                Vt[e] = (t < L && v < V) ? a.qkv[static_cast<size_t>(row0 + t) * a.qkv_stride + a.v_off + h * V + v] : 0.f;
-            }
-            for (int e = tid; e < 3 * C; e += 256) sc[e] = da.scal[idx * 3 * C + e];
-        }
+        stash();
         __syncthreads();
+        if (c + 1 < chunks) fetch(c + 1);
         // K S and Q S for the thread's row
         float ksum[PER], qsum[PER];
 #pragma unroll
         for (int j = 0; j < PER; ++j) ksum[j] = qsum[j] = 0.f;
-        for (int d = 0; d < Dr; ++d) {
-            const float kd = ks[t_row * Dq + d], qd = qs[t_row * Dq + d];
+#pragma unroll 4
+        for (int d = 0; d < Dr; d += 4) {
+            const float4 k4 = *reinterpret_cast<const float4*>(ks + t_row * Dq + d);
+            const float4 q4 = *reinterpret_cast<const float4*>(qs + t_row * Dq + d);
+            const float kd[4] = {k4.x, k4.y, k4.z, k4.w}, qd[4] = {q4.x, q4.y, q4.z, q4.w};
 #pragma unroll
-            for (int j = 0; j < PER; ++j) {
-                const float sv = S[d * 16 + vq + j];
-                ksum[j] += kd * sv;
-                qsum[j] += qd * sv;
+            for (int dd = 0; dd < 4; ++dd) {
+                float sv[PER];
+                read_run<PER>(S + (d + dd) * 16 + vq, sv);
+#pragma unroll
+                for (int j = 0; j < PER; ++j) {
+                    ksum[j] += kd[dd] * sv[j];
+                    qsum[j] += qd[dd] * sv[j];
+                }
             }
         }
         const float gam = sc[t_row], beta = sc[C + t_row];
@@ -225,10 +285,14 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
         float us[PER];
 #pragma unroll
         for (int j = 0; j < PER; ++j) us[j] = 0.f;
-        for (int u = 0; u <= t_row; ++u) {
+        // (T and Aq are zero above the diagonal: a wave walks up to its last row's diagonal, the same for all its lanes)
+#pragma unroll 8
+        for (int u = 0; u < row_bound; ++u) {
             const float w = Tm[t_row * (C + 1) + u];
+            float rv[PER];
+            read_run<PER>(R + u * 16 + vq, rv);
 #pragma unroll
-            for (int j = 0; j < PER; ++j) us[j] += w * R[u * 16 + vq + j];
+            for (int j = 0; j < PER; ++j) us[j] += w * rv[j];
         }
 #pragma unroll
         for (int j = 0; j < PER; ++j) U[t_row * 16 + vq + j] = us[j];
@@ -236,10 +300,13 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
         float os[PER];
 #pragma unroll
         for (int j = 0; j < PER; ++j) os[j] = gam * qsum[j];
-        for (int u = 0; u <= t_row; ++u) {
+#pragma unroll 8
+        for (int u = 0; u < row_bound; ++u) {
             const float w = Aq[t_row * (C + 1) + u];
+            float uv[PER];
+            read_run<PER>(U + u * 16 + vq, uv);
 #pragma unroll
-            for (int j = 0; j < PER; ++j) os[j] += w * U[u * 16 + vq + j];
+            for (int j = 0; j < PER; ++j) os[j] += w * uv[j];
         }
         if (t_row < L) {
 #pragma unroll
@@ -254,10 +321,14 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
             float acc[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) acc[j] = gl * S[d * 16 + half + j];
-            for (int u = 0; u < L; ++u) {
+#pragma unroll 8
+            for (int u = 0; u < C; ++u) {           // (rows behind L hold zeros in U)
                 const float kw = ks[u * Dq + d] * sc[2 * C + u];
+                float uv[8];
+                read_run<4>(U + u * 16 + half, uv);
+                read_run<4>(U + u * 16 + half + 4, uv + 4);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] += kw * U[u * 16 + half + j];
+                for (int j = 0; j < 8; ++j) acc[j] += kw * uv[j];
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) S[d * 16 + half + j] = acc[j];
@@ -290,7 +361,7 @@ static int launch_delta(const DeltaArgs& da, int seqs, int max_q_len, hipStream_
 }
 
 // The requests of the step that bring at least `from` tokens.  Kn, Qn: room for (rows / chunk + requests)
-// chunks of H * chunk * D floats; Tm, Aq: of H * chunk * chunk; scal: of H * 3 * chunk.
+// chunks of H * chunk * (D rounded up to 4) floats; Tm, Aq: of H * chunk * chunk; scal: of H * 3 * chunk.
 extern "C" int pl_delta_chunked(const float* qkv, int qkv_stride, int q_off, int k_off, int v_off,
                                 const float* gates, int gates_stride, int g1_off, int g2_off,
                                 const float* a_log, const float* dt_bias,

@@ -1133,7 +1133,8 @@ def recurrent_scan(kind: str, qkv: torch.Tensor, q_off: int, k_off: int, v_off: 
         tokens = library().pl_recurrent_chunk_tokens(dim)
         chunks = (n // tokens + batch.num_seqs + 1) * heads
         f32 = dict(dtype=torch.float32, device=qkv.device)
-        unit_k, unit_q = torch.empty((chunks, tokens * dim), **f32), torch.empty((chunks, tokens * dim), **f32)
+        padded = (dim + 3) // 4 * 4
+        unit_k, unit_q = torch.empty((chunks, tokens * padded), **f32), torch.empty((chunks, tokens * padded), **f32)
         inverse, masked = torch.empty((chunks, tokens * tokens), **f32), torch.empty((chunks, tokens * tokens), **f32)
         scalars = torch.empty((chunks, 3 * tokens), **f32)
         _check(library().pl_delta_chunked(

@@ -69,7 +69,16 @@ LARGE = model(256, 300, [
     parallel(attention(4, 2, 128, 128, 3, 0.09, (64, 10000.0)), delta(2, 1, 160, 64, 4), 0.8, 0.6, dense(320)),
 ], eps=1e-6, scale=0.3)
 
-CONFIGS = {"odd": ODD, "ones": ONES, "large": LARGE}
+# Eight and sixteen query heads a key head (single tokens then take the attention kernel that makes a group's heads the
+# rows of a tile), heads of 24 in rows of 32, and a model whose first and last layers keep no pages.
+GROUPED = model(64, 150, [
+    lightning(2, 16, 16, (0.95, 0.8)),
+    parallel(attention(8, 1, 32, 32, 3, 0.18, (32, 500.0)), delta(4, 4, 16, 16, 2), 0.7, 0.4, dense(128)),
+    parallel(attention(16, 1, 24, 32, 2, 0.2, (12, 10000.0)), delta(2, 1, 32, 16, 4), 1.0, 0.5),
+    mlstm(2, 16, 32, 5.0, dense(64)),
+], eps=1e-6, scale=2.0)
+
+CONFIGS = {"odd": ODD, "ones": ONES, "large": LARGE, "grouped": GROUPED}
 
 
 def write_model(folder, config, seed=0, dtype="float32", std=0.08, gain_std=0.2, edit=None) -> Path:
@@ -107,4 +116,21 @@ def plain_greedy(folder, prompt, count: int) -> list:
         nxt = int(plain.forward(config, weights, tokens)[-1].argmax())
         out.append(nxt)
         tokens.append(nxt)
+    return out
+
+
+def sensitivity(folder, prompts: dict) -> dict:
+    """name -> a factor a position (>= 1): how much more than the median position this position's logits move when
+    every weight matrix is disturbed by 2^-9 of itself (root mean square over the vocabulary).  Random models have single
+    positions where rounding is amplified ten- to fiftyfold (a read-out near zero before its norm, a score near a
+    tie); a bound on an engine's error there has to grow with it, as the error that rounding alone causes does."""
+    config, weights = load_plain(folder)
+    g = torch.Generator().manual_seed(1234)
+    shaken = {k: v * (1 + (torch.rand(v.shape, generator=g, dtype=v.dtype) - 0.5) * 2.0 ** -8) if v.dim() == 2 and "conv" not in k
+              else v for k, v in weights.items()}
+    out = {}
+    for name, tokens in prompts.items():
+        base = plain.forward(config, weights, tokens)
+        moved = ((plain.forward(config, shaken, tokens) - base) ** 2).mean(-1).sqrt() / base.std()
+        out[name] = torch.clamp(moved / (2 * moved.median()), min=1.0)
     return out

@@ -19,8 +19,9 @@ pytestmark = pytest.mark.gpu
 # Against the plain implementation (64-bit): 32-bit runs are held tightly.  In bfloat16 the rounding of q and k is
 # amplified by softmaxes that these models make sharp on purpose, so such runs get a loose bound there and a tight one
 # against the engine's own whole-prompt run of the same requests (the same roundings; what differs between schedules is
-# the cache, the state and the batch: a lost key or a lost state shows there in full).
-TOLERANCE = {"float32": 1e-4, "bfloat16": 0.15}
+# the cache, the state and the batch: a lost key or a lost state shows there in full).  All bounds are for a position
+# that amplifies rounding as the median position does, and grow with a position's own amplification (``check``).
+TOLERANCE = {"float32": 5e-5, "bfloat16": 0.1}
 BETWEEN_SCHEDULES = 2e-2
 DTYPES = ["float32", "bfloat16"]
 
@@ -39,34 +40,46 @@ def folders(tmp_path_factory):
     def get(name, dtype):
         if (name, dtype) not in made:
             made[name, dtype] = pu.write_model(tmp_path_factory.mktemp(f"papivik_{name}_{dtype}"), pu.CONFIGS[name],
-                                               seed=len(made) + 1, dtype=dtype)
+                                               seed=sorted(pu.CONFIGS).index(name) + 1, dtype=dtype)
         return made[name, dtype]
     return get
 
 
 _whole: dict = {}
+_factor: dict = {}
 
 
 def check(folder, dtype, prompts, steps, live=4, block_size=16, tolerance=None):
+    """Run the steps and hold every wanted row to the plain implementation; a position's bound is the tolerance times
+    how much more than the median position it amplifies rounding (``papivik_util.sensitivity``)."""
     r = replayer(folder, dtype, prompts, live, block_size)
     got = ru.collect(r, steps)
     want = pu.plain_logits(folder, prompts)
-    worst, where = ru.worst_error(got, want)
-    assert worst <= (tolerance or TOLERANCE[dtype]), f"{worst:.3e} at {where}"
+    key = (str(folder), repr(sorted(prompts.items())))
+    if key not in _factor:
+        _factor[key] = pu.sensitivity(folder, prompts)
+    factor = _factor[key]
+    scale = max(float(want[n][p].abs().max()) for (n, p) in got)
+    bound = tolerance or TOLERANCE[dtype]
+    for (n, p), row in got.items():
+        ref = want[n][p].numpy()
+        assert row.shape == ref.shape
+        err = float(np.abs(row.astype(np.float64) - ref).max()) / scale
+        assert err <= bound * float(factor[n][p]), f"{err:.3e} at {(n, p)}, where the bound is {bound * float(factor[n][p]):.3e}"
     assert r.cache.manager.live_sequences == 0 and r.cache.manager.free_state_slots == live, "pages and slots came back"
     if dtype == "bfloat16":
-        key = (str(folder), repr(sorted(prompts.items())))
         if key not in _whole:
             _whole[key] = ru.collect(replayer(folder, dtype, prompts, live), ru.whole(prompts))
-        scale = float(np.mean([want[n][p].std() for (n, p) in got]))
-        # root mean square over the vocabulary.  These random models have single positions where rounding is amplified
-        # tenfold and more (weights disturbed by 2^-9 move the plain implementation's logits by 0.8% at the median
-        # position and by 3 to 35% at the worst), so one position in fifty may be over the bound, none grossly;
-        # a key or a state that a schedule loses is missed by every position behind it.
-        gaps = {at: float(np.sqrt(np.mean((row - _whole[key][at]) ** 2))) / scale for at, row in got.items()}
-        over = {at: gap for at, gap in gaps.items() if gap > BETWEEN_SCHEDULES}
-        assert len(over) <= max(1, len(gaps) // 50) and all(gap <= 0.15 for gap in over.values()), \
-            f"between this schedule and the whole prompt: {sorted(over.items(), key=lambda x: -x[1])[:5]} of {len(gaps)}"
+        spread = float(np.mean([want[n][p].std() for (n, p) in got]))
+        # (One drawn disturbance does not find every position that amplifies rounding: one position in fifty may be over
+        # its bound, none beyond three times it.  A key or a state that a schedule loses is missed by every position behind.)
+        over = {}
+        for (n, p), row in got.items():
+            gap = float(np.sqrt(np.mean((row - _whole[key][(n, p)]) ** 2))) / spread     # root mean square over the vocabulary
+            if gap > BETWEEN_SCHEDULES * float(factor[n][p]):
+                over[n, p] = gap / (BETWEEN_SCHEDULES * float(factor[n][p]))
+        assert len(over) <= max(1, len(got) // 50) and all(x <= 3.0 for x in over.values()), \
+            f"between this schedule and the whole prompt, over the bound by {sorted(over.items(), key=lambda x: -x[1])[:5]} of {len(got)}"
     return r, got
 
 
