@@ -19,12 +19,14 @@ struct DeltaArgs {
     float* scal;     // [chunks, H, 3, C]  G_t; beta_t; G_L / G_t
 };
 
-// PER (4 or 2) neighbouring values of a 16-column row in LDS, in one read (the rows start on 64 bytes).
+// PER (4, 2 or 1) neighbouring values of a row of the column tile in LDS, in one read (the rows start on 32 bytes).
 template <int PER>
 __device__ __forceinline__ void read_run(const float* p, float* out) {
     if (PER == 4) {
         const float4 x = *reinterpret_cast<const float4*>(p);
         out[0] = x.x; out[1] = x.y; out[2] = x.z; out[3] = x.w;
+    } else if (PER == 1) {
+        out[0] = p[0];
     } else {
         const float2 x = *reinterpret_cast<const float2*>(p);
         out[0] = x.x; out[1] = x.y;
@@ -65,21 +67,25 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(DeltaArgs da) {
         qs[e] = q;
         ks[e] = k;
     }
-    if (tid == 0) {
-        const float rate = expf(a.p1[h]), dt_bias = a.p2[h];
-        float sum = 0.f;
-        for (int t = 0; t < C; ++t) {
-            float beta = 0.f;
-            if (t < L) {
-                const float* row = a.gates + static_cast<size_t>(row0 + t) * a.gates_stride;
-                beta = sigmoid_f(row[a.g1_off + h]);
-                sum += -rate * softplus_f(row[a.g2_off + h] + dt_bias);
-            }
-            bs[t] = sum;
-            be[t] = beta;
+    if (tid < C) {
+        // a thread a token: beta, and the logarithm of the decay (summed up below)
+        float beta = 0.f, log_decay = 0.f;
+        if (tid < L) {
+            const float* row = a.gates + static_cast<size_t>(row0 + tid) * a.gates_stride;
+            beta = sigmoid_f(row[a.g1_off + h]);
+            log_decay = -expf(a.p1[h]) * softplus_f(row[a.g2_off + h] + a.p2[h]);
         }
+        bs[tid] = log_decay;
+        be[tid] = beta;
     }
     __syncthreads();
+    if (tid == 255) {
+        float sum = 0.f;
+        for (int t = 0; t < C; ++t) {
+            sum += bs[t];
+            bs[t] = sum;
+        }
+    }
     if (tid < 2 * C) {
         const float* x = (tid < C ? qs : ks) + (tid < C ? tid : tid - C) * Dq;
         float ss = 0.f;
@@ -160,15 +166,15 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(DeltaArgs da) {
     }
 }
 
-// One workgroup: a request, a head, 16 columns of the state; the chunks in order.  What a chunk needs
+// One workgroup: a request, a head, VT (16 or 8) columns of the state; the chunks in order.  What a chunk needs
 // (its unit vectors, T, Aq, the columns of v, the scalars) is asked for while the chunk before is computed
 // and waits in registers: with one workgroup a compute unit nothing else would hide the trip to memory.
-template <int C>
+template <int C, int VT>
 __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
     const ScanArgs& a = da.a;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int D = a.D, V = a.V, H = a.H;
-    const int v0 = blockIdx.x * 16, h = blockIdx.y, s = blockIdx.z;
+    const int v0 = blockIdx.x * VT, h = blockIdx.y, s = blockIdx.z;
     const int slot = a.state_slots[s], n = a.q_len[s];
     if (slot < 0 || n < a.below) return;
     const int chunks = (n + C - 1) / C;
@@ -177,25 +183,26 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
     float* ks = qs + C * Dq;         // [C][Dq]
     float* Tm = ks + C * Dq;         // [C][C + 1]
     float* Aq = Tm + C * (C + 1);    // [C][C + 1]
-    float* S = Aq + C * (C + 1);     // [Dr][16]
-    float* Vt = S + Dr * 16;         // [C][16]
-    float* R = Vt + C * 16;          // [C][16]
-    float* U = R + C * 16;           // [C][16]
-    float* sc = U + C * 16;          // [3][C]
+    float* S = Aq + C * (C + 1);     // [Dr][VT]
+    float* Vt = S + Dr * VT;         // [C][VT]
+    float* R = Vt + C * VT;          // [C][VT]
+    float* U = R + C * VT;           // [C][VT]
+    float* sc = U + C * VT;          // [3][C]
     const int tid = threadIdx.x;
     float* Sg = a.state + static_cast<size_t>(slot) * a.state_stride + a.s_off + static_cast<size_t>(h) * D * V;
-    for (int e = tid; e < Dr * 16; e += 256) {
-        const int d = e / 16, v = v0 + (e & 15);
+    for (int e = tid; e < Dr * VT; e += 256) {
+        const int d = e / VT, v = v0 + e % VT;
         S[e] = (d < D && v < V) ? Sg[static_cast<size_t>(d) * V + v] : 0.f;
     }
     const int first = delta_chunk_number<C>(a, s, 0);
     // a thread's row and columns in the products with C rows: row t, columns vq .. vq + PER - 1
-    constexpr int PER = C == 64 ? 4 : 2;
-    const int t_row = tid / (16 / PER), vq = (tid % (16 / PER)) * PER;
-    const int row_bound = (tid / 64 + 1) * (64 / (16 / PER));      // one past the last row of this thread's wave
+    constexpr int GROUPS = 256 / C, PER = VT / GROUPS;             // threads a row, columns a thread
+    static_assert(PER == 4 || PER == 2 || PER == 1, "a thread takes 4, 2 or 1 columns");
+    const int t_row = tid / GROUPS, vq = (tid % GROUPS) * PER;
+    const int row_bound = (tid / 64 + 1) * (64 / GROUPS);          // one past the last row of this thread's wave
 
     // what a thread fetches of a chunk: up to KQ quads of k and of q, TA quads of T and of Aq, VS values of v
-    constexpr int KQ = 8, TA = C * C / 4 / 256 > 0 ? C * C / 4 / 256 : 1, VS = C * 16 / 256;
+    constexpr int KQ = 8, TA = C * C / 4 / 256 > 0 ? C * C / 4 / 256 : 1, VS = C * VT / 256;
     const int quads_row = Dr / 4, kq_quads = C * quads_row;
     int kq_at[KQ];
 #pragma unroll
@@ -226,7 +233,7 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
         const int L = min(C, n - c * C), row0 = a.q_start[s] + c * C;
 #pragma unroll
         for (int r = 0; r < VS; ++r) {
-            const int e = tid + 256 * r, t = e / 16, v = v0 + (e & 15);
+            const int e = tid + 256 * r, t = e / VT, v = v0 + e % VT;
             vreg[r] = (t < L && v < V) ? a.qkv[static_cast<size_t>(row0 + t) * a.qkv_stride + a.v_off + h * V + v] : 0.f;
         }
         if (tid < 3 * C) sreg = da.scal[idx * 3 * C + tid];
@@ -270,7 +277,7 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
 #pragma unroll
             for (int dd = 0; dd < 4; ++dd) {
                 float sv[PER];
-                read_run<PER>(S + (d + dd) * 16 + vq, sv);
+                read_run<PER>(S + (d + dd) * VT + vq, sv);
 #pragma unroll
                 for (int j = 0; j < PER; ++j) {
                     ksum[j] += kd[dd] * sv[j];
@@ -280,7 +287,7 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
         }
         const float gam = sc[t_row], beta = sc[C + t_row];
 #pragma unroll
-        for (int j = 0; j < PER; ++j) R[t_row * 16 + vq + j] = beta * (Vt[t_row * 16 + vq + j] - gam * ksum[j]);
+        for (int j = 0; j < PER; ++j) R[t_row * VT + vq + j] = beta * (Vt[t_row * VT + vq + j] - gam * ksum[j]);
         __syncthreads();
         float us[PER];
 #pragma unroll
@@ -290,12 +297,12 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
         for (int u = 0; u < row_bound; ++u) {
             const float w = Tm[t_row * (C + 1) + u];
             float rv[PER];
-            read_run<PER>(R + u * 16 + vq, rv);
+            read_run<PER>(R + u * VT + vq, rv);
 #pragma unroll
             for (int j = 0; j < PER; ++j) us[j] += w * rv[j];
         }
 #pragma unroll
-        for (int j = 0; j < PER; ++j) U[t_row * 16 + vq + j] = us[j];
+        for (int j = 0; j < PER; ++j) U[t_row * VT + vq + j] = us[j];
         __syncthreads();
         float os[PER];
 #pragma unroll
@@ -304,7 +311,7 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
         for (int u = 0; u < row_bound; ++u) {
             const float w = Aq[t_row * (C + 1) + u];
             float uv[PER];
-            read_run<PER>(U + u * 16 + vq, uv);
+            read_run<PER>(U + u * VT + vq, uv);
 #pragma unroll
             for (int j = 0; j < PER; ++j) os[j] += w * uv[j];
         }
@@ -314,50 +321,61 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs da) {
                 if (v0 + vq + j < V)
                     a.out[static_cast<size_t>(row0 + t_row) * (H * V) + h * V + v0 + vq + j] = os[j];
         }
-        // S = G_L S + sum_s (G_L / G_s) k_s u_s^T : a thread owns a row d of S and 8 of its 16 columns
+        // S = G_L S + sum_s (G_L / G_s) k_s u_s^T : a thread owns a row d of S and half of its columns
         const float gl = sc[L - 1];
+        constexpr int HALF = VT / 2;
         for (int d = tid / 2; d < Dr; d += 128) {
-            const int half = (tid & 1) * 8;
-            float acc[8];
+            const int half = (tid & 1) * HALF;
+            float acc[HALF];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[j] = gl * S[d * 16 + half + j];
+            for (int j = 0; j < HALF; ++j) acc[j] = gl * S[d * VT + half + j];
 #pragma unroll 8
             for (int u = 0; u < C; ++u) {           // (rows behind L hold zeros in U)
                 const float kw = ks[u * Dq + d] * sc[2 * C + u];
-                float uv[8];
-                read_run<4>(U + u * 16 + half, uv);
-                read_run<4>(U + u * 16 + half + 4, uv + 4);
+                float uv[HALF];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] += kw * uv[j];
+                for (int j = 0; j < HALF; j += 4) read_run<4>(U + u * VT + half + j, uv + j);
+#pragma unroll
+                for (int j = 0; j < HALF; ++j) acc[j] += kw * uv[j];
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) S[d * 16 + half + j] = acc[j];
+            for (int j = 0; j < HALF; ++j) S[d * VT + half + j] = acc[j];
         }
     }
     __syncthreads();
-    for (int e = tid; e < Dr * 16; e += 256) {
-        const int d = e / 16, v = v0 + (e & 15);
+    for (int e = tid; e < Dr * VT; e += 256) {
+        const int d = e / VT, v = v0 + e % VT;
         if (d < D && v < V) Sg[static_cast<size_t>(d) * V + v] = S[e];
     }
+}
+
+template <int C, int VT>
+static int launch_delta_walk(const DeltaArgs& da, int seqs, hipStream_t stream) {
+    const ScanArgs& a = da.a;
+    const int Dr = (a.D + 3) & ~3, Dq = Dr + 4;
+    const size_t lds_w = (2 * static_cast<size_t>(C) * Dq + 2 * C * (C + 1) + Dr * VT + 3 * C * VT + 3 * C) * sizeof(float);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&delta_walk_kernel<C, VT>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_w));
+    PL_REQUIRE(e == hipSuccess, "delta_chunked: %zu bytes of LDS refused: %s", lds_w, hipGetErrorString(e));
+    delta_walk_kernel<C, VT><<<dim3(pl_ceil_div(a.V, VT), a.H, seqs), 256, lds_w, stream>>>(da);
+    PL_CHECK_LAUNCH("delta_chunked (walk)");
+    return 0;
 }
 
 template <int C>
 static int launch_delta(const DeltaArgs& da, int seqs, int max_q_len, hipStream_t stream) {
     const ScanArgs& a = da.a;
-    const int Dq = ((a.D + 3) & ~3) + 4, Dr = (a.D + 3) & ~3;
+    const int Dq = ((a.D + 3) & ~3) + 4;
     const size_t lds_p = (2 * static_cast<size_t>(C) * Dq + C * (C + 1) + 4 * C) * sizeof(float);
-    const size_t lds_w = (2 * static_cast<size_t>(C) * Dq + 2 * C * (C + 1) + Dr * 16 + 3 * C * 16 + 3 * C) * sizeof(float);
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&delta_prepare_kernel<C>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_p));
     PL_REQUIRE(e == hipSuccess, "delta_chunked: %zu bytes of LDS refused: %s", lds_p, hipGetErrorString(e));
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&delta_walk_kernel<C>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_w));
-    PL_REQUIRE(e == hipSuccess, "delta_chunked: %zu bytes of LDS refused: %s", lds_w, hipGetErrorString(e));
     delta_prepare_kernel<C><<<dim3(pl_ceil_div(max_q_len, C), a.H, seqs), 256, lds_p, stream>>>(da);
     PL_CHECK_LAUNCH("delta_chunked (prepare)");
-    delta_walk_kernel<C><<<dim3(pl_ceil_div(a.V, 16), a.H, seqs), 256, lds_w, stream>>>(da);
-    PL_CHECK_LAUNCH("delta_chunked (walk)");
-    return 0;
+    // A request's chunks are a chain, so the walk has heads x tiles of columns workgroups a request and no more:
+    // tiles of 8 columns where tiles of 16 would leave half of the chip's compute units without one.
+    if (a.H * pl_ceil_div(a.V, 16) * 2 <= pl_compute_units()) return launch_delta_walk<C, 8>(da, seqs, stream);
+    return launch_delta_walk<C, 16>(da, seqs, stream);
 }
 
 // The requests of the step that bring at least `from` tokens.  Kn, Qn: room for (rows / chunk + requests)

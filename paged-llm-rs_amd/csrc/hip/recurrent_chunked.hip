@@ -25,23 +25,27 @@ struct ChunkArgs {
 template <int C>
 __device__ __forceinline__ int chunk_number(const ScanArgs& a, int s, int c) { return a.q_start[s] / C + s + c; }
 
-// The gates of the tokens of one chunk: a (log decay) summed up to b, and g = w - b.  One thread.
+// The gates of the tokens of one chunk, a thread a token: a (log decay) into b, w (log weight of the write) into g.
+// `sum_gates` then turns b into its running sum and g into w - b.
 template <int KIND>
-__device__ void chunk_gates(const ScanArgs& a, int h, int row0, int L, float* b, float* g) {
-    float sum = 0.f;
+__device__ __forceinline__ void token_gates(const ScanArgs& a, int h, int row, float* b, float* g) {
     if (KIND == PL_SCAN_LIGHTNING) {
-        const float la = logf(a.p1[h]);
-        for (int t = 0; t < L; ++t) { sum += la; b[t] = sum; g[t] = -sum; }
+        *b = logf(a.p1[h]);
+        *g = 0.f;
     } else {
-        const float bias_i = a.p1[h], bias_f = a.p2[h];
-        for (int t = 0; t < L; ++t) {
-            const float* row = a.gates + static_cast<size_t>(row0 + t) * a.gates_stride;
-            const float gi = a.cap * tanhf((row[a.g1_off + h] + bias_i) / a.cap);
-            const float gf = logsigmoid_f(a.cap * tanhf((row[a.g2_off + h] + bias_f) / a.cap));
-            sum += gf;
-            b[t] = sum;
-            g[t] = gi - sum;
-        }
+        const float* gates = a.gates + static_cast<size_t>(row) * a.gates_stride;
+        *g = a.cap * tanhf((gates[a.g1_off + h] + a.p1[h]) / a.cap);
+        *b = logsigmoid_f(a.cap * tanhf((gates[a.g2_off + h] + a.p2[h]) / a.cap));
+    }
+}
+
+// One thread, after a barrier behind token_gates.
+__device__ __forceinline__ void sum_gates(int L, float* b, float* g) {
+    float sum = 0.f;
+    for (int t = 0; t < L; ++t) {
+        sum += b[t];
+        b[t] = sum;
+        g[t] -= sum;
     }
 }
 
@@ -82,8 +86,10 @@ __global__ __launch_bounds__(256) void chunk_summary_kernel(ChunkArgs ca) {
         if (KIND == PL_SCAN_LIGHTNING) v = silu_f(v);
         vs[e] = v;
     }
+    if (tid < L) token_gates<KIND>(a, h, row0 + tid, bs + tid, ws + tid);
+    __syncthreads();
     if (tid == 0) {
-        chunk_gates<KIND>(a, h, row0, L, bs, ws);
+        sum_gates(L, bs, ws);
         const float end = bs[L - 1];
         float most = ws[0];
         for (int t = 1; t < L; ++t) most = fmaxf(most, ws[t]);
@@ -220,20 +226,20 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(ChunkArgs ca) {
         }
         vs[e] = v;
     }
+    if (tid < L) token_gates<KIND>(a, h, row0 + tid, bs + tid, gs + tid);
+    __syncthreads();
     if (tid == 0) {
-        chunk_gates<KIND>(a, h, row0, L, bs, gs);
-        if (KIND == PL_SCAN_LIGHTNING) {
-            for (int t = 0; t < L; ++t) es[t] = expf(bs[t]);
-        } else {
-            const float m0 = ca.scal[idx * 4 + 2];
-            float top = m0;
+        sum_gates(L, bs, gs);
+        if (KIND == PL_SCAN_MLSTM) {
+            float top = ca.scal[idx * 4 + 2];
             for (int t = 0; t < L; ++t) {
                 top = fmaxf(top, gs[t]);
                 cm[t] = top;
-                es[t] = expf(m0 - top);
             }
         }
     }
+    __syncthreads();
+    if (tid < L) es[tid] = KIND == PL_SCAN_LIGHTNING ? expf(bs[tid]) : expf(ca.scal[idx * 4 + 2] - cm[tid]);
     __syncthreads();
     const int ty = tid / 16, tx = tid % 16;
     {

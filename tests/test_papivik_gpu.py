@@ -93,6 +93,7 @@ ALONE = {
     "attention": pu.parallel(pu.attention(6, 3, 24, 40, 3, 0.25, (12, 300.0)), pu.delta(2, 1, 16, 16, 2), 1.0, 0.0),
     "attention, no rotation, one tap": pu.parallel(pu.attention(2, 1, 40, 24, 1, 0.5), pu.delta(2, 1, 16, 16, 2), 1.0, 0.0),
     "delta": pu.parallel(pu.attention(2, 1, 16, 16, 2, 0.5), pu.delta(6, 2, 24, 40, 4), 0.0, 1.0),
+    "delta, many columns": pu.parallel(pu.attention(2, 1, 16, 16, 2, 0.5), pu.delta(16, 4, 16, 144, 2), 0.0, 1.0),
     "delta, one tap": pu.parallel(pu.attention(2, 1, 16, 16, 2, 0.5), pu.delta(2, 2, 72, 80, 1), 0.0, 1.0),
     "feed-forward": pu.lightning(1, 16, 16, (0.9,), pu.dense(136)),
 }
