@@ -219,7 +219,7 @@ extern "C" int pl_recurrent_scan(int kind, const float* qkv, int qkv_stride, int
 
 // ---------------------------------------------------------------------------
 // Short causal convolution over time, a filter a channel:
-//   y[t, c] = sum_j w[c, j] * u[t - taps + 1 + j, c]
+//   y[t, c] = sum_j w[j, c] * u[t - taps + 1 + j, c]      (w is stored a tap a row)
 // u are the columns [off, off + C) of the rows; the taps - 1 rows before a request's first row of the
 // step come from its history hist[taps - 1][C] (zeros at a request's start), the last one the newest.
 // ---------------------------------------------------------------------------
@@ -232,7 +232,7 @@ __device__ __forceinline__ float conv_at(const float* __restrict__ rows, int str
         const int src = r - back;
         const float u = src >= 0 ? rows[static_cast<size_t>(row - back) * stride + off + c]
                                  : hist[static_cast<size_t>(taps - 1 + src) * C + c];
-        acc += w[c * taps + jt] * u;
+        acc += w[jt * C + c] * u;
     }
     return acc;
 }
@@ -310,18 +310,34 @@ __global__ __launch_bounds__(64) void gated_group_norm_kernel(const float* __res
                                                               int gate_off, int act, T* __restrict__ out) {
     const int t = blockIdx.x, first = blockIdx.y * group;
     const float* row = x + static_cast<size_t>(t) * width + first;
+    // a lane keeps up to eight of its values between the sum and the output (groups up to 512 are read once)
+    constexpr int KEEP = 8;
+    float kept[KEEP];
     float ss = 0.f;
-    for (int e = threadIdx.x; e < group; e += 64) ss += row[e] * row[e];
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        const int e = threadIdx.x + 64 * k;
+        kept[k] = e < group ? row[e] : 0.f;
+        ss += kept[k] * kept[k];
+    }
+    for (int e = threadIdx.x + 64 * KEEP; e < group; e += 64) ss += row[e] * row[e];
     ss = wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / static_cast<float>(group) + eps);
-    for (int e = threadIdx.x; e < group; e += 64) {
-        const int c = first + e;
-        float y = row[e] * inv * gain[c % gain_len];
-        if (act >= 0) {
-            const float z = gate[static_cast<size_t>(t) * gate_stride + gate_off + c];
-            y *= act == 0 ? sigmoid_f(z) : silu_f(z);
+    const float* g = gate != nullptr ? gate + static_cast<size_t>(t) * gate_stride + gate_off + first : nullptr;
+    T* o = out + static_cast<size_t>(t) * width + first;
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        const int e = threadIdx.x + 64 * k;
+        if (e < group) {
+            float y = kept[k] * inv * gain[(first + e) % gain_len];
+            if (act >= 0) y *= act == 0 ? sigmoid_f(g[e]) : silu_f(g[e]);
+            o[e] = from_float<T>(y);
         }
-        out[static_cast<size_t>(t) * width + c] = from_float<T>(y);
+    }
+    for (int e = threadIdx.x + 64 * KEEP; e < group; e += 64) {
+        float y = row[e] * inv * gain[(first + e) % gain_len];
+        if (act >= 0) y *= act == 0 ? sigmoid_f(g[e]) : silu_f(g[e]);
+        o[e] = from_float<T>(y);
     }
 }
 

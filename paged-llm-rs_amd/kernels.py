@@ -1162,7 +1162,7 @@ def _conv_args(rows, off, weight, history, batch):
     _need(weight, "convolution filters", None, torch.float32)
     if rows.dim() != 2 or weight.dim() != 2:
         raise TensorError(f"rows of shape {tuple(rows.shape)}, filters of shape {tuple(weight.shape)}")
-    channels, taps = weight.shape
+    taps, channels = weight.shape
     if not 1 <= taps <= 16 or off < 0 or off + channels > rows.shape[1]:
         raise TensorError(f"{channels} channels of {taps} taps from column {off} of rows of {rows.shape[1]}")
     history, stride = _state_view(history, "the convolution's history")
@@ -1174,8 +1174,9 @@ def _conv_args(rows, off, weight, history, batch):
 
 def short_conv(rows: torch.Tensor, off: int, weight: torch.Tensor, history: torch.Tensor, batch,
                silu: bool = False, out: torch.Tensor | None = None) -> torch.Tensor:
-    """y[t, c] = sum_j weight[c, j] * u[t - taps + 1 + j, c] over the columns [off, off + channels) of
-    ``rows``; the rows before a request's first of this step come from ``history`` [slots, (taps-1) * channels]
+    """y[t, c] = sum_j weight[j, c] * u[t - taps + 1 + j, c] over the columns [off, off + channels) of
+    ``rows`` (``weight`` is [taps, channels]: a checkpoint's [channels, taps] transposed, so that neighbouring
+    channels' values of a tap are neighbours in memory); the rows before a request's first of this step come from ``history`` [slots, (taps-1) * channels]
     (newest last, zeros at a request's start), which is left as it is: ``conv_history`` moves it afterwards."""
     n, channels, taps, history, stride = _conv_args(rows, off, weight, history, batch)
     if out is None:

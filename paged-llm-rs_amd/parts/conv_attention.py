@@ -57,7 +57,7 @@ class ConvAttention:
         self.proj = Linear.fused([params["q"], params["k"], params["v"]])
         self.channels = H * D + G * D + G * V
         f32 = lambda t: t.to(torch.float32).contiguous()
-        self.conv_w = torch.cat([f32(params["q.conv"]), f32(params["k.conv"]), f32(params["v.conv"])], 0).contiguous()
+        self.conv_w = torch.cat([f32(params["q.conv"]), f32(params["k.conv"]), f32(params["v.conv"])], 0).t().contiguous()   # [taps, channels]
         if spec.qk_norm_eps is not None:
             self.q_gain, self.k_gain, self.eps = f32(params["q.norm"]), f32(params["k.norm"]), float(spec.qk_norm_eps)
         else:

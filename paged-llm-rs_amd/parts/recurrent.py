@@ -140,7 +140,7 @@ class GatedDelta(_ScanMixer):
         self.H, self.G, self.D, self.V = spec.num_heads, spec.num_qk_heads, spec.head_dim, spec.value_dim
         self._fuse(params, ["q", "k", "v", "g", "b", "a"])       # q | k | v first: the convolution's channels
         self.channels = 2 * self.G * self.D + self.H * self.V
-        self.conv_w = torch.cat([_f32(params["q.conv"]), _f32(params["k.conv"]), _f32(params["v.conv"])], 0).contiguous()
+        self.conv_w = torch.cat([_f32(params["q.conv"]), _f32(params["k.conv"]), _f32(params["v.conv"])], 0).t().contiguous()   # [taps, channels]
         self.o_proj = Linear(params["o"])
         self.gain = _f32(params["norm"])
         self.a_log, self.dt_bias = _f32(params["A_log"]), _f32(params["dt_bias"])
