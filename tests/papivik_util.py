@@ -78,7 +78,15 @@ GROUPED = model(64, 150, [
     mlstm(2, 16, 32, 5.0, dense(64)),
 ], eps=1e-6, scale=2.0)
 
-CONFIGS = {"odd": ODD, "ones": ONES, "large": LARGE, "grouped": GROUPED}
+# Head sizes that are no multiple of 4 (30, 22) or of 8 (20, 36, 44), a rotation over 10 values, a width that is a
+# multiple of 4 only, seven taps.
+UNEVEN = model(52, 75, [
+    parallel(attention(3, 1, 30, 20, 7, 0.21, (10, 123.0)), delta(4, 2, 22, 36, 3), 0.9, 1.1, dense(44)),
+    lightning(3, 30, 20, (0.7, 0.93, 0.99)),
+    mlstm(2, 22, 44, 9.0),
+], eps=3e-6, scale=0.8)
+
+CONFIGS = {"odd": ODD, "ones": ONES, "large": LARGE, "grouped": GROUPED, "uneven": UNEVEN}
 
 
 def write_model(folder, config, seed=0, dtype="float32", std=0.08, gain_std=0.2, edit=None) -> Path:

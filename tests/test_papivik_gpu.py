@@ -160,6 +160,16 @@ def test_unequal_requests_together_with_pages_and_slots_used_again(folders, name
     check(folders(name, dtype), dtype, prompts, ru.mixed(prompts, seed=seed))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["odd", "large", "uneven"])
+def test_portions_at_the_edges_of_the_chunked_kernels(folders, name, dtype):
+    """Portions one token short of, exactly at and one token past what the kernels cut by: 16 tokens (below it a request
+    goes token by token), chunks of 64 tokens (32 for heads above 128) and twice that; then single tokens again."""
+    prompts = ru.make_prompts(pu.CONFIGS[name]["vocab"], [15 + 16 + 17 + 63 + 64 + 65 + 31 + 32 + 33 + 127 + 128 + 129 + 3, 70], seed=14)
+    sizes = (15, 16, 17, 63, 64, 65, 31, 32, 33, 127, 128, 129, 1, 1, 1)
+    check(folders(name, dtype), dtype, prompts, ru.portions(prompts, sizes=sizes))
+
+
 def test_schedules_agree_with_each_other_in_32_bit(folders):
     """Whole, decoded and in portions: the same request gives the same logits but for rounding."""
     folder = folders("odd", "float32")
