@@ -301,18 +301,41 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(ChunkArgs ca) {
         }
     }
     const float* S0 = ca.Sin + idx * D * V;
-    int col[4];
+    if (C == 64) {
+        // The tile of S_0 (D rows of 64 columns) goes through LDS, where k lay (nobody reads k behind the barrier
+        // above, and C rows of Dq hold D rows of 64): all its loads are on their way at once.
+        float* St = ks;
+        for (int e = tid; e < D * 64; e += 256) {
+            const int d = e / 64, v = vt * 64 + (e & 63);
+            St[e] = v < V ? S0[static_cast<size_t>(d) * V + v] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int d = 0; d < D; ++d) {
+            float sv[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) col[j] = min(vt * 64 + tx + 16 * j, V - 1);
-    for (int d = 0; d < D; ++d) {
-        float sv[4];
+            for (int j = 0; j < 4; ++j) sv[j] = St[d * 64 + tx + 16 * j];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) sv[j] = S0[static_cast<size_t>(d) * V + col[j]];
+            for (int i = 0; i < TT; ++i) {
+                const float q = qs[(ty + 16 * i) * Dq + d];
 #pragma unroll
-        for (int i = 0; i < TT; ++i) {
-            const float q = qs[(ty + 16 * i) * Dq + d];
+                for (int j = 0; j < 4; ++j) before[i][j] += q * sv[j];
+            }
+        }
+    } else {
+        int col[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) before[i][j] += q * sv[j];
+        for (int j = 0; j < 4; ++j) col[j] = min(vt * 64 + tx + 16 * j, V - 1);
+        for (int d = 0; d < D; ++d) {
+            float sv[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sv[j] = S0[static_cast<size_t>(d) * V + col[j]];
+#pragma unroll
+            for (int i = 0; i < TT; ++i) {
+                const float q = qs[(ty + 16 * i) * Dq + d];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) before[i][j] += q * sv[j];
+            }
         }
     }
     __syncthreads();
