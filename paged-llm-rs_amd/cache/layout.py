@@ -20,10 +20,13 @@ from ..errors import ConfigError
 @dataclass(frozen=True)
 class KVCacheSpec:
     """Keys and values of ``kv_heads`` heads of ``head_dim``; with a window only
-    the last ``window`` positions are ever read."""
+    the last ``window`` positions are ever read.  ``values_in_keys``: a token's values are read out of
+    its row of keys (a layer that keeps one small vector a token and rebuilds both from it), so the layer
+    has one pool, which stands in the place of both."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    values_in_keys: bool = False
 
 
 @dataclass(frozen=True)
@@ -95,7 +98,8 @@ class CacheLayout:
     def bytes_per_token(self, element_size: int) -> int:
         """Bytes of keys and values one token takes over all layers
         (reference: batch.rs:43-46)."""
-        return sum(2 * len(g.layers) * g.spec.kv_heads * g.spec.head_dim * element_size for g in self.groups)
+        return sum((1 if g.spec.values_in_keys else 2) * len(g.layers) * g.spec.kv_heads * g.spec.head_dim * element_size
+                   for g in self.groups)
 
     def blocks_within(self, budget_bytes: int, block_size: int, element_size: int) -> int:
         """Pages a byte budget holds, at least one (reference: batch.rs:54-57)."""

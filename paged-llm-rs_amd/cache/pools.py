@@ -44,10 +44,10 @@ class PagedCache:
         for g in layout.groups:
             width = g.spec.kv_heads * g.spec.head_dim
             for layer in g.layers:
-                self._pools[layer] = (
-                    torch.zeros((num_blocks * block_size, width), dtype=dtype, device=self.device),
-                    torch.zeros((num_blocks * block_size, width), dtype=dtype, device=self.device),
-                )
+                keys = torch.zeros((num_blocks * block_size, width), dtype=dtype, device=self.device)
+                # (a layer whose values are read out of its keys' rows has the one pool in both places)
+                values = keys if g.spec.values_in_keys else torch.zeros_like(keys)
+                self._pools[layer] = (keys, values)
         self._states = {
             layer: torch.zeros((max_seqs, *spec.shape), dtype=spec.dtype, device=self.device)
             for layer, spec in layout.states.items()
@@ -55,7 +55,7 @@ class PagedCache:
 
     @property
     def bytes(self) -> int:
-        return sum(k.numel() * k.element_size() * 2 for k, _ in self._pools.values())
+        return sum(k.numel() * k.element_size() * (1 if v is k else 2) for k, v in self._pools.values())
 
     def layer_view(self, layer: int, batch) -> LayerKV:
         if layer not in self._pools:

@@ -9,6 +9,7 @@ from __future__ import annotations
 from pathlib import Path
 
 from ..errors import ConfigError, UnsupportedError
+from .lefavik import LefavikConfig
 from .papivik import PapivikConfig
 from .qwen3 import Qwen3Config, read_json
 
@@ -64,3 +65,4 @@ def load_config(source):
 
 register_architecture("Qwen3ForCausalLM", Qwen3Config, model_type="qwen3")
 register_architecture("Papivik", PapivikConfig, model_type="papivik")
+register_architecture("Lefavik", LefavikConfig, model_type="lefavik")

@@ -50,6 +50,8 @@ class GatedMlpSpec:
     kind: str = "gated_mlp"
     intermediate_size: int = 0
     activation: str = "silu"
+    # the tensors' names inside the feed-forward, where a family stores them under others: (gate, up, down)
+    names: Optional[tuple] = None
 
 
 @dataclass(frozen=True)
@@ -164,3 +166,50 @@ class DenseMlpSpec:
     kind: str = "dense_mlp"
     intermediate_size: int = 0
     activation: str = "gelu_tanh"
+
+
+# ---- attention with sinks, distance penalties and keys rebuilt from a small vector --------------------
+
+@dataclass(frozen=True)
+class SinkAttentionSpec:
+    """Grouped-query softmax attention over a paged cache whose softmax has one more term in its denominator
+    (a sink: a score without a key or a value), with optional extras: q and k divided by their root mean
+    square over a head (no gain), a query temperature that grows with the logarithm of the position, a
+    penalty a head on the distance between query and key, and a window."""
+    kind: str = "sink_attention"
+    num_heads: int = 0
+    num_kv_heads: int = 0
+    head_dim: int = 0
+    value_dim: int = 0
+    scale: Optional[float] = None           # None = 1/sqrt(head_dim)
+    qk_unit_eps: Optional[float] = None     # None: q and k are used as projected
+    # q at position p times 1 + coef * ln(floor((p + 1) / every) + 1); None: no temperature
+    temperature_coef: Optional[float] = None
+    temperature_every: int = 1
+    # score_ij -= slope_h (i - j); "geometric": slope_h = 2^(-slope_span (h + 1) / heads); None: no penalty
+    distance_slopes: Optional[str] = None
+    slope_span: float = 8.0
+    window: Optional[int] = None            # keys j with i - window < j <= i; None: all keys up to i
+    sink: Optional[str] = "zero"            # "zero": a sink of score 0; "learned": one a head (tensor ``sink``); None
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values of all heads are rebuilt from one small vector a token (``kv_rank``
+    values, normalised) and whose heads share one rotated key part of ``rotary_dim`` values: the pages hold
+    those two and nothing else.  A query head is [head_dim values that are not rotated | rotary_dim rotated]."""
+    kind: str = "latent_attention"
+    num_heads: int = 0
+    head_dim: int = 0                       # the unrotated part of a query/key head
+    rotary_dim: int = 0                     # the rotated part, shared by the heads on the key side
+    value_dim: int = 0
+    kv_rank: int = 0
+    rotary_turned: int = 0                  # how many values of the rotated part turn (pairs 2i, 2i + 1)
+    rotary_base: float = 10000.0
+    max_positions: int = 0                  # rows of the rotation's tables
+    scale: Optional[float] = None           # None = 1/sqrt(head_dim + rotary_dim)
+    norm_eps: float = 1e-6                  # of the norm on the small vector
+    sink: Optional[str] = "learned"         # as in SinkAttentionSpec
+    gated: bool = True                      # a head's read-out times sigmoid(gate projection of the layer's input)
+    window: Optional[int] = None
+    borrows: bool = False                   # no projection onto the small vector: the schedule names the layer whose pages are read

@@ -14,7 +14,11 @@
 template <typename T, typename OUT>
 __global__ void __launch_bounds__(256)
 gemm_nt_kernel(const T* __restrict__ x, const T* __restrict__ w, OUT* __restrict__ y, int n, int N,
-               int K, int ldx, int ldy) {
+               int K, int ldx, int ldy, long sx = 0, long sw = 0, long sy = 0) {
+    // (a batch of products, one a blockIdx.z: operands and result `sx`, `sw`, `sy` elements further on)
+    x += blockIdx.z * sx;
+    w += blockIdx.z * sw;
+    y += blockIdx.z * sy;
     // Tiles are stored k-major so that the inner loop reads consecutive LDS words.
     __shared__ float xs[TILE_K][TILE_M + 4];
     __shared__ float ws[TILE_K][TILE_N + 4];
@@ -87,5 +91,33 @@ extern "C" int pl_gemm_plain(const void* x, const void* w, void* y, int n, int N
         PL_REQUIRE(false, "gemm: dtype code %d", dtype);
     }
     PL_CHECK_LAUNCH("gemm_plain");
+    return 0;
+}
+
+// A product a head: y[t, h, 0:N] = x[t, h, 0:K] . w[h]^T with w [heads, N, K]; head h of a row of x begins
+// `sx` elements behind head h - 1 (rows `ldx` apart), of y `sy` elements (rows `ldy` apart).  The same sums in
+// the same order as the single product above.
+extern "C" int pl_gemm_heads(const void* x, const void* w, void* y, int n, int heads, int N, int K, int ldx,
+                             long sx, int ldy, long sy, int dtype, int out_f32, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && heads > 0 && heads <= 65535 && N > 0 && K > 0 && ldx >= K && ldy >= N && sx >= 0 && sy >= 0,
+               "gemm over heads: %d rows, %d heads of %d x %d, row strides %d and %d", n, heads, N, K, ldx, ldy);
+    if (n == 0) return 0;
+    dim3 grid(pl_ceil_div(N, TILE_N), pl_ceil_div(n, TILE_M), heads);
+    PL_REQUIRE(grid.y <= 65535, "gemm over heads: %d rows are more than one launch covers", n);
+    const long sw = static_cast<long>(N) * K;
+    if (dtype == PL_DTYPE_F32) {
+        gemm_nt_kernel<float, float><<<grid, 256, 0, stream>>>(
+            static_cast<const float*>(x), static_cast<const float*>(w), static_cast<float*>(y), n, N, K, ldx, ldy, sx, sw, sy);
+    } else if (dtype == PL_DTYPE_BF16) {
+        if (out_f32)
+            gemm_nt_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(
+                static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<float*>(y), n, N, K, ldx, ldy, sx, sw, sy);
+        else
+            gemm_nt_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>(
+                static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(y), n, N, K, ldx, ldy, sx, sw, sy);
+    } else {
+        PL_REQUIRE(false, "gemm over heads: dtype code %d", dtype);
+    }
+    PL_CHECK_LAUNCH("gemm_heads");
     return 0;
 }

@@ -35,7 +35,12 @@ def _signatures(lib) -> None:
         "pl_qk_norm_rope_kv_write": [p, p, p, i, f, p, p, i, p, p, p, i, i, p, p, i, i, i, i, i, i, i, p],
         "pl_swiglu": [p, p, i, i, i, i, p],
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
-        "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
+        "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p, p, p],
+        "pl_gemm_heads": [p, p, p, i, i, i, i, i, ctypes.c_long, i, ctypes.c_long, i, i, p],
+        "pl_head_prepare": [p, i, i, i, f, p, p, p, p, i, i, i, i, f, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, i, p],
+        "pl_latent_prepare": [p, i, i, i, p, f, p, p, i, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, i, p],
+        "pl_head_gate": [p, i, p, i, i, p, i, i, i, p],
+        "pl_add_position_rows": [p, p, i, p, i, i, i, p],
         "pl_paged_attention_prefill_tile": [i, i],
         "pl_argmax": [p, p, p, p, i, i, p],
         "pl_sample": [p, p, p, p, p, p, i, i, i, p],
@@ -268,13 +273,23 @@ def gemm_plain(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None
     return out
 
 
+def _head_numbers(t, what: str, heads: int):
+    """A 32-bit number a query head (sinks, slopes), or None."""
+    if t is None:
+        return None
+    return _need(t, what, (heads,), torch.float32)
+
+
 def paged_attention_plain(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, positions: torch.Tensor,
                           seq_of: torch.Tensor, block_table: torch.Tensor, block_size: int,
                           k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int,
-                          scale: float, window: int = 0) -> torch.Tensor:
+                          scale: float, window: int = 0, sinks: torch.Tensor | None = None,
+                          slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of every token over the keys 0..position of its request, read
     through the block table.  ``q`` is the fused projection buffer whose rows begin
-    with the nq*d query values."""
+    with the nq*d query values.  ``slopes`` [nq]: slope_h * (i - j) is taken off the score of key j for
+    the query at position i.  ``sinks`` [nq]: exp(sink_h) joins the softmax's denominator, once, unscaled
+    and without a value.  Key and value pool may be the same tensor."""
     n = positions.numel()
     _need(q, "query buffer")
     if q.dim() != 2 or q.shape[0] != n or q.shape[1] != q_row_stride or q_row_stride < nq * d:
@@ -287,10 +302,11 @@ def paged_attention_plain(q: torch.Tensor, q_row_stride: int, out: torch.Tensor,
         _need(pool, what, None, q.dtype)
         if pool.dim() != 2 or pool.shape[1] != nkv * d or pool.shape[0] % block_size != 0:
             raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{block_size}, {nkv * d}]")
+    sinks, slopes = _head_numbers(sinks, "sinks", nq), _head_numbers(slopes, "distance slopes", nq)
     _check(library().pl_paged_attention_plain(
         q.data_ptr(), q_row_stride, out.data_ptr(), positions.data_ptr(), seq_of.data_ptr(),
         block_table.data_ptr(), block_table.shape[1], block_size, k_pool.data_ptr(), v_pool.data_ptr(),
-        n, nq, nkv, d, float(scale), int(window or 0), _code(q, "query buffer"), _stream()))
+        n, nq, nkv, d, float(scale), int(window or 0), _code(q, "query buffer"), _ptr(sinks), _ptr(slopes), _stream()))
     return out
 
 
@@ -1296,3 +1312,136 @@ def weighted_sum_(x: torch.Tensor, a: float, y: torch.Tensor, b: float) -> torch
     _need(y, "second branch", tuple(x.shape), torch.float32)
     _check(library().pl_weighted_sum(x.data_ptr(), float(a), y.data_ptr(), float(b), x.numel(), _stream()))
     return x
+
+
+# ---- attention layers with sinks, distance penalties, and pages that hold one small vector a token -------------
+
+def gemm_heads(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """A product a head: out[t, h, :N] = x[t, h, :K] . w[h]^T, w [heads, N, K].  ``x`` [n, heads, >= K] and ``out``
+    [n, heads, >= N] may be views whose rows and heads lie further apart than their own sizes (the last axis
+    contiguous); a view's values behind K or N are neither read nor written.  In 32-bit on the vector units
+    (sums in ascending k: the true 32-bit path); in bfloat16 the library's batched product on the matrix cores."""
+    heads, N, K = w.shape
+    _need(w, "weights a head")
+    n = x.shape[0]
+    if x.dim() != 3 or out.dim() != 3 or x.shape[1] != heads or out.shape[1] != heads or out.shape[0] != n:
+        raise TensorError(f"a product a head of {tuple(x.shape)} with {tuple(w.shape)} into {tuple(out.shape)}")
+    if x.shape[2] != K or out.shape[2] != N or x.stride(2) != 1 or out.stride(2) != 1:
+        raise TensorError(f"a product a head of {tuple(x.shape)} with {tuple(w.shape)} into {tuple(out.shape)}")
+    if not x.is_cuda or x.dtype != w.dtype or out.dtype != w.dtype:
+        raise TensorError("a product a head needs its operands on the GPU and of one type")
+    if n == 0:
+        return out
+    if w.dtype == torch.bfloat16 and n > GEMM_HEADS_PLAIN_ROWS:
+        torch.bmm(x.transpose(0, 1), w.transpose(1, 2), out=out.transpose(0, 1))
+        return out
+    _check(library().pl_gemm_heads(x.data_ptr(), w.data_ptr(), out.data_ptr(), n, heads, N, K, x.stride(0), x.stride(1),
+                                   out.stride(0), out.stride(1), _code(w, "weights a head"), 0, _stream()))
+    return out
+
+
+# Up to this many rows a bfloat16 product a head runs on the vector units (one small launch); above, the library's.
+GEMM_HEADS_PLAIN_ROWS = 0
+
+
+def head_prepare(rows: torch.Tensor, off: int, batch, kv, q_out: torch.Tensor, H: int, G: int, D: int, V: int,
+                 padded: int, unit_eps: float | None = None, q_gain=None, k_gain=None, cos=None, sin=None,
+                 rot_off: int = 0, rot: int = 0, temperature: tuple | None = None, write_kv: bool = True) -> None:
+    """Between an attention layer's projections and the attention kernels: ``rows`` [n, >= off + H D + G D + G V]
+    (32-bit) holds q | k | v from column ``off``.  q and k are divided by their root mean square over a head
+    (``unit_eps``; times a gain where one is given), ``rot`` values from ``rot_off`` on turn in pairs (2i, 2i + 1)
+    by the tables' angles, q is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) (``temperature`` =
+    (coef, every)); q goes to ``q_out`` [n, H * padded], k and v into the pages, every head in ``padded`` values."""
+    n = rows.shape[0]
+    _need(rows, "projected rows", None, torch.float32)
+    if rows.dim() != 2:
+        raise TensorError(f"projected rows of shape {tuple(rows.shape)}")
+    _need(q_out, "query buffer", (n, H * padded))
+    for pool, what in ((kv.k_pool, "key pool"), (kv.v_pool, "value pool")):
+        _need(pool, what, None, q_out.dtype)
+        if pool.dim() != 2 or pool.shape[1] != G * padded or pool.shape[0] % kv.block_size:
+            raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{kv.block_size}, {G * padded}]")
+    for g, what in ((q_gain, "query gain"), (k_gain, "key gain")):
+        if g is not None:
+            _need(g, what, (D,), torch.float32)
+    table_rows = 0
+    if rot:
+        _need(cos, "cosine table", None, torch.float32)
+        _need(sin, "sine table", tuple(cos.shape), torch.float32)
+        if cos.dim() != 2 or cos.shape[1] != rot // 2:
+            raise TensorError(f"rotary tables have shape {tuple(cos.shape)}, expected [positions, {rot // 2}]")
+        table_rows = cos.shape[0]
+    coef, every = temperature if temperature is not None else (0.0, 1)
+    _check(library().pl_head_prepare(
+        rows.data_ptr(), rows.shape[1], int(off), 1 if unit_eps is not None else 0, float(unit_eps or 0.0),
+        _ptr(q_gain), _ptr(k_gain), _ptr(cos) if rot else 0, _ptr(sin) if rot else 0, int(rot_off), int(rot), table_rows,
+        1 if temperature is not None else 0, float(coef), int(every), batch.positions.data_ptr(),
+        batch.seq_of.data_ptr(), kv.block_table.data_ptr(), kv.block_table.shape[1], kv.block_size,
+        1 if write_kv else 0, q_out.data_ptr(), kv.k_pool.data_ptr(), kv.v_pool.data_ptr(),
+        _code(q_out, "query buffer"), n, H, G, D, V, padded, _stream()))
+
+
+def latent_prepare(rows: torch.Tensor, q_off: int, kv_off: int, gain, eps: float, cos, sin, turned: int, batch, kv,
+                   q_plain: torch.Tensor, q_out: torch.Tensor, H: int, D: int, rot: int, R: int, padded: int,
+                   write_kv: bool = True) -> None:
+    """For a layer whose pages hold one small vector a token.  ``rows`` (32-bit): H query heads of [D | rot] from
+    column ``q_off``; the small vector's R values and the rotated key part's ``rot`` from ``kv_off``.  The
+    unrotated query parts go head-major into ``q_plain`` [H, n, D]; the rotated parts, turned, into values
+    R .. R + rot of every head of ``q_out`` [n, H * padded] with zeros behind them; with ``write_kv`` the
+    token's row of the pages becomes [norm(vector) * gain | turned key part | zeros]."""
+    n = rows.shape[0]
+    _need(rows, "projected rows", None, torch.float32)
+    _need(q_out, "query buffer", (n, H * padded))
+    _need(q_plain, "unrotated query parts", (H, n, D), q_out.dtype)
+    pool = kv.k_pool
+    _need(pool, "pages", None, q_out.dtype)
+    if pool.dim() != 2 or pool.shape[1] != padded or pool.shape[0] % kv.block_size:
+        raise TensorError(f"pages have shape {tuple(pool.shape)}, expected [pages*{kv.block_size}, {padded}]")
+    if write_kv:
+        _need(gain, "gain of the small vector", (R,), torch.float32)
+    table_rows = 0
+    if turned:
+        _need(cos, "cosine table", None, torch.float32)
+        _need(sin, "sine table", tuple(cos.shape), torch.float32)
+        if cos.dim() != 2 or cos.shape[1] != turned // 2:
+            raise TensorError(f"rotary tables have shape {tuple(cos.shape)}, expected [positions, {turned // 2}]")
+        table_rows = cos.shape[0]
+    _check(library().pl_latent_prepare(
+        rows.data_ptr(), rows.shape[1], int(q_off), int(kv_off), _ptr(gain) if write_kv else 0, float(eps),
+        _ptr(cos) if turned else 0, _ptr(sin) if turned else 0, int(turned), table_rows, batch.positions.data_ptr(),
+        batch.seq_of.data_ptr(), kv.block_table.data_ptr(), kv.block_table.shape[1], kv.block_size,
+        1 if write_kv else 0, q_plain.data_ptr(), q_out.data_ptr(), pool.data_ptr(), _code(q_out, "query buffer"),
+        n, H, D, rot, R, padded, _stream()))
+
+
+def head_gate_(x: torch.Tensor, rows: torch.Tensor, off: int, positions, H: int, V: int) -> torch.Tensor:
+    """x[t, h, :] *= sigmoid(rows[t, off + h]) in place; ``x`` [n, H * V], ``rows`` 32-bit."""
+    n = x.shape[0]
+    _need(x, "read-outs", (n, H * V))
+    _need(rows, "gate rows", None, torch.float32)
+    if rows.dim() != 2 or rows.shape[0] != n or rows.shape[1] < off + H:
+        raise TensorError(f"gate rows of shape {tuple(rows.shape)} for {n} tokens and {H} gates from column {off}")
+    _check(library().pl_head_gate(x.data_ptr(), _code(x, "read-outs"), rows.data_ptr(), rows.shape[1], int(off),
+                                  _ptr(positions), n, H, V, _stream()))
+    return x
+
+
+def add_position_rows_(x: torch.Tensor, table: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+    """x[t] += table[positions[t]] on the 32-bit stream; rows at position -1 stay as they are."""
+    n, width = x.shape
+    _need(x, "stream", None, torch.float32)
+    _need(table, "position table")
+    if table.dim() != 2 or table.shape[1] != width:
+        raise TensorError(f"a position table of shape {tuple(table.shape)} for a stream of width {width}")
+    _need(positions, "positions", (n,), torch.int32)
+    _check(library().pl_add_position_rows(x.data_ptr(), table.data_ptr(), _code(table, "position table"),
+                                          positions.data_ptr(), n, width, table.shape[0], _stream()))
+    return x
+
+
+def sink_attention(q: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int, scale: float,
+                   window: int = 0, sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
+    """Attention for every token of a step with a sink a head in the softmax's denominator and a penalty a
+    head on the distance; ``q`` [n, nq * d] holds the prepared queries."""
+    return paged_attention_plain(q, q.shape[1], out, batch.positions, batch.seq_of, kv.block_table, kv.block_size,
+                                 kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, sinks=sinks, slopes=slopes)

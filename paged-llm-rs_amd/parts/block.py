@@ -201,3 +201,75 @@ class SublayerNormBlock:
 
 
 register_block("sublayer_norm", SublayerNormBlock)
+
+
+class SharedNormBlock:
+    """The arrangement with one norm a layer, read by both sublayers: with n = norm1(x),
+    x <- x + mixer(n) + feed_forward(n).  A layer whose spec has no feed-forward adds the mixer's output only.
+
+    The stream is 32-bit and every sum into it is: a sublayer's last product adds its 32-bit sums into the
+    stream itself where its kernel can, and hands them back 32-bit to be added here where it cannot.
+    Tensor names: the norm's gain is stored under the norm's own name."""
+
+    NAMES = {"norm1": "norm1", "mixer": "mix", "feed_forward": "mlp"}
+
+    @classmethod
+    def names_of(cls, layer) -> dict:
+        given = getattr(layer, "names", None) or {}
+        unknown = sorted(set(given) - set(cls.NAMES))
+        if unknown:
+            raise ConfigError(f"a layer names members that this arrangement does not have: {unknown}")
+        return {**cls.NAMES, **given}
+
+    @classmethod
+    def declare(cls, layer, hidden: int) -> list:
+        from ..weights.loader import ParamDecl
+
+        n = cls.names_of(layer)
+        mixer = lookup(MIXERS, layer.mixer.kind, "mixer")
+        decls = [ParamDecl(n["norm1"], (hidden,), "gain")] + prefixed(mixer.declare(layer.mixer, hidden), n["mixer"])
+        if layer.feed_forward is not None:
+            ffn = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")
+            decls += prefixed(ffn.declare(layer.feed_forward, hidden), n["feed_forward"])
+        return decls
+
+    def __init__(self, layer, hidden: int, params: dict, dtype, device, shared: dict):
+        n = self.names = self.names_of(layer)
+        norm = lookup(NORMS, layer.norm.kind, "norm")
+        self.dtype = dtype
+        self.norm1 = norm(layer.norm, hidden, {"weight": params[n["norm1"]]}, dtype, device)
+        self.mixer = lookup(MIXERS, layer.mixer.kind, "mixer")(
+            layer.mixer, hidden, scoped(params, n["mixer"]), dtype, device, shared)
+        self.feed_forward = None
+        if layer.feed_forward is not None:
+            self.feed_forward = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")(
+                layer.feed_forward, hidden, scoped(params, n["feed_forward"]), dtype, device, shared)
+
+    @property
+    def graph_safe(self) -> bool:
+        return getattr(self.mixer, "graph_safe", True) and getattr(self.feed_forward, "graph_safe", True)
+
+    @property
+    def first_norm(self):
+        return self.norm1
+
+    def forward(self, resid, delta, ctx):
+        # (the norm's rows are written out: two sublayers read them, and the first adds into the stream
+        # before the second runs)
+        rows = self.norm1.apply(resid, delta, self.dtype)
+        ctx.residual = resid
+        mixed = self.mixer.forward(rows, ctx)
+        ctx.residual = None
+        if mixed is not None:
+            kernels.residual_add(resid, mixed)
+        if self.feed_forward is not None:
+            if getattr(self.feed_forward, "fuses", False):
+                out = self.feed_forward.forward(rows, residual=resid, out_dtype=torch.float32)
+            else:
+                out = self.feed_forward.forward(rows)
+            if out is not None:
+                kernels.residual_add(resid, out)
+        return None
+
+
+register_block("shared_norm", SharedNormBlock)

@@ -13,19 +13,29 @@ from .registry import register_feed_forward
 
 
 class GatedMlp:
-    @staticmethod
-    def declare(spec, hidden: int) -> list:
+    NAMES = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
+
+    @classmethod
+    def names_of(cls, spec) -> tuple:
+        names = getattr(spec, "names", None) or cls.NAMES
+        if len(names) != 3:
+            raise UnsupportedError(f"a gated feed-forward has three tensors (gate, up, down), the spec names {len(names)}")
+        return tuple(names)
+
+    @classmethod
+    def declare(cls, spec, hidden: int) -> list:
         i = spec.intermediate_size
-        return [ParamDecl("gate_proj.weight", (i, hidden)), ParamDecl("up_proj.weight", (i, hidden)),
-                ParamDecl("down_proj.weight", (hidden, i))]
+        gate, up, down = cls.names_of(spec)
+        return [ParamDecl(gate, (i, hidden)), ParamDecl(up, (i, hidden)), ParamDecl(down, (hidden, i))]
 
     def __init__(self, spec, hidden: int, params: dict, dtype, device, shared: dict):
         if spec.activation not in kernels.ACTIVATIONS:
             raise UnsupportedError(f"activation {spec.activation!r}, the kernels know {', '.join(sorted(kernels.ACTIVATIONS))}")
         self.activation = spec.activation
+        gate, up, down = self.names_of(spec)
         # one product for gate and up: the output row is [gate | up]
-        self.gate_up_proj = Linear.fused([params["gate_proj.weight"], params["up_proj.weight"]])
-        self.down_proj = Linear(params["down_proj.weight"])
+        self.gate_up_proj = Linear.fused([params[gate], params[up]])
+        self.down_proj = Linear(params[down])
 
     # forward takes a norm still to run in place of rows, and may add its result into the stream
     fuses = True
@@ -34,7 +44,7 @@ class GatedMlp:
     # ... and room for the norm that follows the stream, which the product that adds into it may fill
     hands_forward = True
 
-    def forward(self, x, residual: torch.Tensor | None = None, trace=None, hand=None):
+    def forward(self, x, residual: torch.Tensor | None = None, trace=None, hand=None, out_dtype=None):
         """``x``: normalised rows, or a PendingNorm.  With ``residual`` (the 32-bit stream) the
         result is added there where the product kernel can do it, and None comes back; ``hand``
         (``kernels.HandedNorm``) is then filled where that kernel can leave the next norm's work behind."""
@@ -50,7 +60,9 @@ class GatedMlp:
             return out
         # (few rows: the activation is the product's epilogue)
         act = self.gate_up_proj.forward(x, swiglu=True, activation=self.activation)
-        return self.down_proj.forward(act, add_into=residual, hand=hand if residual is not None else None)
+        # (``out_dtype``: the type of what comes back where the product could not add it into the stream itself)
+        return self.down_proj.forward(act, out_dtype=out_dtype, add_into=residual,
+                                      hand=hand if residual is not None else None)
 
 
 register_feed_forward("gated_mlp", GatedMlp)

@@ -16,7 +16,7 @@ from ..cache.layout import CacheLayout
 from ..config import load_config
 from ..errors import ConfigError, UnsupportedError, WeightError
 from ..weights.loader import ParamDecl, load_weights
-from . import attention, block, conv_attention, mlp, norm, parallel, recurrent, transforms  # noqa: F401  (register the built-in parts)
+from . import attention, block, conv_attention, latent_attention, mlp, norm, parallel, recurrent, sink_attention, transforms  # noqa: F401  (register the built-in parts)
 from .linear import Linear, linears_of
 from .norm import PendingNorm
 from .registry import BLOCKS, EMBED_TRANSFORMS, LOGIT_TRANSFORMS, NORMS, lookup, prefixed, scoped
@@ -26,14 +26,29 @@ DTYPES = {"float32": torch.float32, "f32": torch.float32, "bfloat16": torch.bflo
           torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
 
 
+class TransformChain:
+    """Several transforms applied one after the other, where a spec names a list of them."""
+
+    def __init__(self, members: list):
+        self.members = members
+        self.graph_safe = all(getattr(m, "graph_safe", True) for m in members)
+
+    def __call__(self, x, batch):
+        for member in self.members:
+            x = member(x, batch)
+        return x
+
+
 def _transforms(spec) -> list:
-    """(attribute, class) of the transforms the spec names: of the stream behind the embedding and of the logits."""
+    """(attribute, classes) of the transforms the spec names: of the stream behind the embedding and of the
+    logits.  A spec names one transform or a list of them, applied in that order."""
     found = []
     for key, registry, what in (("embed_transform", EMBED_TRANSFORMS, "embedding transform"),
                                 ("logit_transform", LOGIT_TRANSFORMS, "logit transform")):
         kind = (spec.extra or {}).get(key)
         if kind is not None:
-            found.append((key, lookup(registry, kind, what)))
+            kinds = kind if isinstance(kind, (list, tuple)) else (kind,)
+            found.append((key, [lookup(registry, k, what) for k in kinds]))
     return found
 
 
@@ -64,9 +79,10 @@ def declare_parameters(spec) -> list:
     decls += _final_norm_decls(spec, final)
     # A tied checkpoint may still store the output projection; the stored tensor wins.
     decls.append(ParamDecl(spec.head_name, (spec.vocab_size, spec.hidden_size), "matrix", optional=True))
-    for _, cls in _transforms(spec):
-        if hasattr(cls, "declare"):
-            decls += list(cls.declare(spec))
+    for _, classes in _transforms(spec):
+        for cls in classes:
+            if hasattr(cls, "declare"):
+                decls += list(cls.declare(spec))
     return decls
 
 
@@ -134,8 +150,9 @@ class DecoderModel:
             raise WeightError(f"no {spec.head_name}, and the config does not tie the embeddings")
         self.lm_head = Linear(head)
         self.embed_transform = self.logit_transform = None
-        for key, cls in _transforms(spec):
-            setattr(self, key, cls(spec, params, dtype, self.device))
+        for key, classes in _transforms(spec):
+            members = [cls(spec, params, dtype, self.device) for cls in classes]
+            setattr(self, key, members[0] if len(members) == 1 else TransformChain(members))
         for entry in spec.schedule:
             if not 0 <= entry.layer < len(self.blocks):
                 raise ConfigError(f"the schedule names layer {entry.layer} of {len(self.blocks)}")

@@ -1,0 +1,110 @@
+"""Grouped-query softmax attention over the paged cache with a sink in the softmax's denominator and,
+as the spec asks, q and k as unit vectors (divided by their root mean square over a head, no gain), a
+query temperature that grows with the logarithm of the position, a penalty a head on the distance
+between query and key, and a window.
+
+weights_ij = exp(s_ij) / (exp(sink_h) + sum over the visible j of exp(s_ij)),
+s_ij = scale (q_i . k_j) - slope_h (i - j); a sink has no key and no value, so a row's weights sum to
+less than one.  One kernel stands between the projection and the attention kernel (unit vectors,
+temperature, queries out, keys and values into the pages), all in 32-bit from the projection's 32-bit
+sums, one rounding at the store.  Query/key heads and value heads may differ in size: every head is
+stored in a row of ``padded`` values with zeros behind its own, and the output projection's columns are
+padded alike once, at load.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import kernels
+from ..cache.layout import KVCacheSpec
+from ..errors import UnsupportedError
+from ..weights.loader import ParamDecl
+from .linear import Linear
+from .registry import register_mixer
+
+
+def head_sinks(kind, heads: int, params: dict, device):
+    """The sink of every head as 32-bit numbers: zeros, the tensor ``sink``, or None where there is none."""
+    if kind is None:
+        return None
+    if kind == "zero":
+        return torch.zeros((heads,), dtype=torch.float32, device=device)
+    if kind == "learned":
+        return params["sink"].to(torch.float32).contiguous()
+    raise UnsupportedError(f"a sink of kind {kind!r} (zero, learned or none)")
+
+
+def head_slopes(kind, heads: int, span: float, device):
+    """The distance penalty of every head: ``geometric`` is 2^(-span (h + 1) / heads)."""
+    if kind is None:
+        return None
+    if kind != "geometric":
+        raise UnsupportedError(f"distance slopes of kind {kind!r} (geometric or none)")
+    return torch.tensor([2.0 ** (-span * (h + 1) / heads) for h in range(heads)], dtype=torch.float64).to(
+        torch.float32).to(device)
+
+
+class SinkAttention:
+    graph_safe = True
+    short_portion = kernels.SHORT_PORTION
+
+    @staticmethod
+    def declare(spec, hidden: int) -> list:
+        H, G, D, V = spec.num_heads, spec.num_kv_heads, spec.head_dim, spec.value_dim
+        decls = [ParamDecl("q", (H * D, hidden)), ParamDecl("k", (G * D, hidden)), ParamDecl("v", (G * V, hidden)),
+                 ParamDecl("o", (hidden, H * V))]
+        if spec.sink == "learned":
+            decls.append(ParamDecl("sink", (H,), "bias"))
+        return decls
+
+    def __init__(self, spec, hidden: int, params: dict, dtype, device, shared: dict):
+        H, G, D, V = spec.num_heads, spec.num_kv_heads, spec.head_dim, spec.value_dim
+        if H < 1 or G < 1 or H % G:
+            raise UnsupportedError(f"{H} query heads over {G} key heads, which do not group evenly")
+        unit = 1 if dtype == torch.float32 else 16       # the bfloat16 attention kernels take head sizes in 16s
+        self.padded = (max(D, V) + unit - 1) // unit * unit
+        if not 1 <= self.padded <= 1024:
+            raise UnsupportedError(f"heads of {D} and {V}: the attention kernels take head sizes up to 1024")
+        if spec.temperature_coef is not None and spec.temperature_every < 1:
+            raise UnsupportedError(f"a query temperature every {spec.temperature_every} positions")
+        self.spec, self.dtype = spec, dtype
+        self.H, self.G, self.D, self.V = H, G, D, V
+        self.scale = float(spec.scale) if spec.scale is not None else 1.0 / math.sqrt(D)
+        self.window = int(spec.window or 0)
+        self.proj = Linear.fused([params["q"], params["k"], params["v"]])
+        self.sinks = head_sinks(spec.sink, H, params, device)
+        self.slopes = head_slopes(spec.distance_slopes, H, float(spec.slope_span), device)
+        self.temperature = ((float(spec.temperature_coef), int(spec.temperature_every))
+                            if spec.temperature_coef is not None else None)
+        w_o = params["o"]
+        if self.padded != V:
+            wide = torch.zeros((hidden, H, self.padded), dtype=w_o.dtype, device=w_o.device)
+            wide[:, :, :V] = w_o.view(hidden, H, V)
+            w_o = wide.view(hidden, H * self.padded)
+        self.o_proj = Linear(w_o)
+
+    def cache_spec(self):
+        return KVCacheSpec(self.G, self.padded, self.window or None)
+
+    def state_spec(self):
+        return None
+
+    def forward(self, x, ctx):
+        """``x``: the normed rows.  The output comes back as 32-bit sums, or None where the output projection
+        added them into ``ctx.residual`` itself."""
+        batch, kv = ctx.batch, ctx.kv()
+        rows = self.proj.forward(x, out_dtype=torch.float32)
+        n = rows.shape[0]
+        q = torch.empty((n, self.H * self.padded), dtype=self.dtype, device=rows.device)
+        kernels.head_prepare(rows, 0, batch, kv, q, self.H, self.G, self.D, self.V, self.padded,
+                             unit_eps=self.spec.qk_unit_eps, temperature=self.temperature, write_kv=ctx.writes_cache)
+        out = torch.empty((n, self.H * self.padded), dtype=self.dtype, device=rows.device)
+        kernels.sink_attention(q, out, batch, kv, self.H, self.G, self.padded, self.scale, self.window,
+                               sinks=self.sinks, slopes=self.slopes)
+        return self.o_proj.forward(out, out_dtype=torch.float32, add_into=getattr(ctx, "residual", None))
+
+
+register_mixer("sink_attention", SinkAttention)

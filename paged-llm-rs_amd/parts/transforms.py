@@ -2,8 +2,12 @@
 
 from __future__ import annotations
 
+import torch
+
 from .. import kernels
-from .registry import register_embed_transform
+from ..errors import ConfigError
+from ..weights.loader import ParamDecl
+from .registry import NORMS, lookup, register_embed_transform, register_logit_transform
 
 
 class EmbeddingScale:
@@ -19,3 +23,62 @@ class EmbeddingScale:
 
 
 register_embed_transform("scale", EmbeddingScale)
+
+
+class LearnedPosition:
+    """x[t] <- x[t] + table[position of t]: a learned vector a position, added to the 32-bit stream unscaled.
+    The table's checkpoint name is ``extra["position_table_name"]``; it has ``max_positions`` rows."""
+
+    graph_safe = True
+
+    @staticmethod
+    def declare(spec) -> list:
+        return [ParamDecl(spec.extra["position_table_name"], (spec.max_positions, spec.hidden_size), "embedding")]
+
+    def __init__(self, spec, params: dict, dtype, device):
+        self.table = params[spec.extra["position_table_name"]]
+
+    def __call__(self, x, batch):
+        return kernels.add_position_rows_(x, self.table, batch.positions)
+
+
+class StreamNorm:
+    """x <- norm(x) on the stream right behind the embedding; the norm is ``extra["stream_norm"]`` (a NormSpec),
+    its gain the tensor ``extra["stream_norm_name"]``."""
+
+    graph_safe = True
+
+    @staticmethod
+    def declare(spec) -> list:
+        norm = lookup(NORMS, spec.extra["stream_norm"].kind, "norm")
+        decls = norm.declare(spec.extra["stream_norm"], spec.hidden_size)
+        if len(decls) != 1:
+            raise ConfigError(f"a norm of {len(decls)} tensors cannot be stored under one name")
+        return [ParamDecl(spec.extra["stream_norm_name"], decls[0].shape, decls[0].role)]
+
+    def __init__(self, spec, params: dict, dtype, device):
+        norm = lookup(NORMS, spec.extra["stream_norm"].kind, "norm")
+        local = norm.declare(spec.extra["stream_norm"], spec.hidden_size)[0].name
+        self.norm = norm(spec.extra["stream_norm"], spec.hidden_size, {local: params[spec.extra["stream_norm_name"]]},
+                         dtype, device)
+
+    def __call__(self, x, batch):
+        # (the normalised rows in 32-bit are the stream from here on)
+        return self.norm.apply(x, None, torch.float32)
+
+
+class LogitScale:
+    """logits <- logits * extra["logit_scale"]."""
+
+    graph_safe = True
+
+    def __init__(self, spec, params: dict, dtype, device):
+        self.scale = float(spec.extra["logit_scale"])
+
+    def __call__(self, logits, batch):
+        return kernels.scale_(logits, self.scale) if self.scale != 1.0 and logits.numel() else logits
+
+
+register_embed_transform("learned_position", LearnedPosition)
+register_embed_transform("stream_norm", StreamNorm)
+register_logit_transform("scale", LogitScale)
