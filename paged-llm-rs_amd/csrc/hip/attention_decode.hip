@@ -209,7 +209,8 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
                               const int* __restrict__ block_table, int max_blocks, int block_size,
                               bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool, int nq,
                               int nkv, int d, float scale_log2e, int window, int splits, int tiles, int g,
-                              uint32_t splits_magic, ad_fuse_t fuse) {
+                              uint32_t splits_magic, ad_fuse_t fuse, const float* __restrict__ sinks,
+                              const float* __restrict__ slopes) {
     constexpr int KPW = PL_WAVE / LPK;  // keys a wave handles with one load
     constexpr int ROUND = WV * KPW * U;
     extern __shared__ float lds[];      // [AD_PAGES_LDS] page numbers, then [WV][GT][2] running max and sum, [WV][GT][d] accumulators
@@ -352,6 +353,11 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
             for (int w = 0; w < 4; ++w) qp[hq].v[w] = real ? qraw[hq].v[w] : 0u;
         }
     }
+    // (a penalty on the distance, where the layer has one: slope_h (pos - j) leaves the score, in the exponent's unit)
+    const bool tilted = slopes != nullptr;
+    float tilt[GT];
+#pragma unroll
+    for (int hq = 0; hq < GT; ++hq) tilt[hq] = tilted ? slopes[h0 + min(hq, heads - 1)] * 1.4426950408889634f : 0.f;
     float m[GT], l[GT], acc[GT][8];
 #pragma unroll
     for (int hq = 0; hq < GT; ++hq) {
@@ -400,16 +406,19 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     // Values are taken two keys at a time: element i of both keys in one word against both probabilities
     // (rounded to bfloat16, as the matrix-core kernels round them), one instruction an element and head.
     static_assert(U % 2 == 0, "values are taken two keys at a time");
-    auto consume = [&](u32x4* kraw, u32x4* vraw, const bool* ok) {
+    auto consume = [&](u32x4* kraw, u32x4* vraw, const bool* ok, int round) {
         float s[U][GT];
+        const int base = s_begin + round * ROUND + wave * KPW * U;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
+            const float far = static_cast<float>(pos - (base + u * KPW + sub));
 #pragma unroll
             for (int hq = 0; hq < GT; ++hq) {
                 float dot = 0.f;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) dot = ad_dot2(qp[hq].v[w], kraw[u].v[w], dot);
                 dot = key_sum<LPK>(dot) * scale_log2e;
+                if (tilted) dot = fmaf(-tilt[hq], far, dot);
                 s[u][hq] = ok[u] ? dot : -INFINITY;
             }
             const uint32_t keep = ok[u] ? 0xffffffffu : 0u;
@@ -454,10 +463,10 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
         }
     };
     for (int r = 0; r < rounds; r += 2) {
-        consume(ka, va, oka);
+        consume(ka, va, oka, r);
         if (r + 2 < rounds) ask(r + 2, ka, va, oka);
         if (r + 1 < rounds) {
-            consume(kb, vb, okb);
+            consume(kb, vb, okb, r + 1);
             if (r + 3 < rounds) ask(r + 3, kb, vb, okb);
         }
     }
@@ -507,6 +516,14 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
         }
         const int h = h0 + hq;
         if (splits == 1) {
+            if (sinks != nullptr) {
+                // a sink: one more term of the denominator, unscaled, with no value behind it
+                const float sk = sinks[h] * 1.4426950408889634f;
+                const float top = fmaxf(big, sk);
+                const float keep = big == -INFINITY ? 0.f : exp2f(big - top);
+                sum = sum * keep + exp2f(sk - top);
+                a *= keep;
+            }
             out[(static_cast<size_t>(t) * nq + h) * d + dd] = from_float<bf16_t>(sum > 0.f ? a / sum : 0.f);
         } else {
             const size_t pi = (static_cast<size_t>(t) * nq + h) * splits + split;
@@ -530,7 +547,7 @@ __global__ void __launch_bounds__(256)
 paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                              bf16_t* __restrict__ out, const int* __restrict__ positions,
                              const int* __restrict__ seq_of, const int* __restrict__ q_len, int short_limit,
-                             int nq, int d, int splits, int n, int num_seqs) {
+                             int nq, int d, int splits, int n, int num_seqs, const float* __restrict__ sinks) {
     const int per_token = nq * d;
     int t, rest;
     bool inside;
@@ -570,6 +587,13 @@ paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __
         sum = fmaf(ls[s], w, sum);
         a = fmaf(as[s], w, a);
     }
+    if (sinks != nullptr) {
+        const float sk = sinks[h] * 1.4426950408889634f;
+        const float top = fmaxf(big, sk);
+        const float keep = big == -INFINITY ? 0.f : exp2f(big - top);
+        sum = sum * keep + exp2f(sk - top);
+        a *= keep;
+    }
     out[(static_cast<size_t>(t) * nq + h) * d + dd] = from_float<bf16_t>(sum > 0.f ? a / sum : 0.f);
 }
 
@@ -580,7 +604,7 @@ static int launch_decode_keys(const void* q, int q_stride, void* out, float* par
                               const int* positions, const int* seq_of, const int* q_len, int short_limit, int num_seqs,
                               int short_rows, const int* block_table, int max_blocks, int block_size, void* k_pool,
                               void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
-                              const ad_fuse_t& fuse, hipStream_t stream) {
+                              const ad_fuse_t& fuse, const float* sinks, const float* slopes, hipStream_t stream) {
     constexpr int WV = AD_WAVES;
     const int g = nq / nkv;
     const int tiles = pl_ceil_div(g, GT);
@@ -599,14 +623,14 @@ static int launch_decode_keys(const void* q, int q_stride, void* out, float* par
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), part_acc, part_ml, positions, seq_of,
         q_len, short_limit, compact ? num_seqs : 0, block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool),
         static_cast<bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles, g,
-        static_cast<uint32_t>((0x100000000ull + splits - 1) / static_cast<unsigned>(splits)), fuse);
+        static_cast<uint32_t>((0x100000000ull + splits - 1) / static_cast<unsigned>(splits)), fuse, sinks, slopes);
     PL_CHECK_LAUNCH("paged_attention_decode");
     if (splits > 1) {
         const dim3 mgrid = dim3(pl_ceil_div(nq * d, 256), compact ? short_rows : n);
 #define AD_MERGE(SP)                                                                                              \
     paged_attention_merge_kernel<SP><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, static_cast<bf16_t*>(out),     \
                                                                 positions, seq_of, q_len, short_limit, nq, d,     \
-                                                                splits, n, compact ? num_seqs : 0)
+                                                                splits, n, compact ? num_seqs : 0, sinks)
         if (splits <= 4) AD_MERGE(4);
         else if (splits <= 8) AD_MERGE(8);
         else if (splits <= 16) AD_MERGE(16);
@@ -629,12 +653,12 @@ static int launch_decode(const void* q, int q_stride, void* out, float* part_acc
                          const int* positions, const int* seq_of, const int* q_len, int short_limit, int num_seqs,
                          int short_rows, const int* block_table, int max_blocks, int block_size, void* k_pool,
                          void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
-                         const ad_fuse_t& fuse, hipStream_t stream) {
+                         const ad_fuse_t& fuse, const float* sinks, const float* slopes, hipStream_t stream) {
     const long long workgroups = static_cast<long long>(nkv) * pl_ceil_div(nq / nkv, GT) * n * splits;
 #define AD_KEYS_CALL(U)                                                                                            \
     return launch_decode_keys<LPK, GT, U>(q, q_stride, out, part_acc, part_ml, positions, seq_of, q_len,          \
                                           short_limit, num_seqs, short_rows, block_table, max_blocks, block_size,  \
-                                          k_pool, v_pool, n, nq, nkv, d, scale, window, splits, fuse, stream)
+                                          k_pool, v_pool, n, nq, nkv, d, scale, window, splits, fuse, sinks, slopes, stream)
     if constexpr (GT <= 2) {
         if (workgroups <= pl_compute_units()) AD_KEYS_CALL(8);
         AD_KEYS_CALL(4);
@@ -649,11 +673,11 @@ static int dispatch_gt(int gt, const void* q, int q_stride, void* out, float* pa
                        const int* positions, const int* seq_of, const int* q_len, int short_limit, int num_seqs,
                        int short_rows, const int* block_table, int max_blocks, int block_size, void* k_pool,
                        void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
-                       const ad_fuse_t& fuse, hipStream_t stream) {
+                       const ad_fuse_t& fuse, const float* sinks, const float* slopes, hipStream_t stream) {
 #define AD_CALL(G)                                                                                              \
     return launch_decode<LPK, G>(q, q_stride, out, part_acc, part_ml, positions, seq_of, q_len, short_limit,   \
                                  num_seqs, short_rows, block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale,    \
-                                 window, splits, fuse, stream)
+                                 window, splits, fuse, sinks, slopes, stream)
     switch (gt) {
         case 1: AD_CALL(1);
         case 2: AD_CALL(2);
@@ -679,7 +703,7 @@ extern "C" int pl_paged_attention_decode(const void* q, int q_stride, void* out,
                                          void* v_pool, int n, int nq, int nkv, int d, float scale, int window,
                                          int splits, int fuse_mode, const void* q_gain, const void* k_gain,
                                          int gain_dtype, float eps, const float* cos_table, const float* sin_table,
-                                         int rot, hipStream_t stream) {
+                                         int rot, const float* sinks, const float* slopes, hipStream_t stream) {
     PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "decode attention: head size %d, which has to be a multiple of 16 up to 256", d);
     PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "decode attention: %d query heads over %d key heads", nq, nkv);
     PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0 && splits >= 1 && splits <= AD_MAX_SPLITS,
@@ -703,7 +727,7 @@ extern "C" int pl_paged_attention_decode(const void* q, int q_stride, void* out,
 #define AD_LPK(L)                                                                                                  \
     return dispatch_gt<L>(gt, q, q_stride, out, part_acc, part_ml, positions, seq_of, q_len, short_limit,        \
                           num_seqs, short_rows, block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale, window,      \
-                          splits, fuse, stream)
+                          splits, fuse, sinks, slopes, stream)
     if (chunks <= 2) AD_LPK(2);
     if (chunks <= 4) AD_LPK(4);
     if (chunks <= 8) AD_LPK(8);

@@ -177,7 +177,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                                int block_size, const bf16_t* __restrict__ k_pool,
                                const bf16_t* __restrict__ v_pool, int nq, int nkv, int d, float scale_log2e,
                                int window, int total_work, int splits, float* __restrict__ part_acc,
-                               float* __restrict__ part_ml, int compact) {
+                               float* __restrict__ part_ml, int compact, const float* __restrict__ sinks,
+                               const float* __restrict__ slopes) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
     constexpr int NT = 64 * NW * KS;
@@ -262,6 +263,10 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
             qf[kk].raw = ap_u32x4{{0u, 0u, 0u, 0u}};
     }
     const int q_pos = start + wq;                               // position of this lane's query
+    // A penalty on the distance, where the layer has one: slope_h (i - j) leaves the score.  The running maximum is
+    // kept on raw scores, so the penalty enters in their unit (divided by the scale).
+    const bool tilted = slopes != nullptr;
+    const float tilt = tilted ? slopes[q_head] * 1.4426950408889634f / scale_log2e : 0.f;
     const int wave_first = GR ? q_pos : start + q0 + wave * 32; // position of the wave's first query
     const int wave_last = GR ? q_pos : start + min(q0 + wave * 32 + 31, count - 1);
     const bool wave_active = GR ? wave * 32 < group : q0 + wave * 32 < count;
@@ -610,10 +615,18 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     };
     auto soften = [&](int k0, bool masked) {
         float mx = -INFINITY;
+        // Key k0 + c + 4*h, c a constant of the register, is seen by this lane's query iff c <= reach
+        // (and c > reach - window); it stands reach - c positions before the query.
+        const int reach = q_pos - k0 - 32 * kt0 - 4 * h;
+        if (tilted) {
+            const float from = -tilt * static_cast<float>(reach);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    s[kt][r] += fmaf(tilt, static_cast<float>(32 * kt + 8 * (r >> 2) + (r & 3)), from);
+        }
         if (masked) {
-            // Key k0 + c + 4*h, c a constant of the register, is seen by this lane's query iff c <= reach
-            // (and c > reach - window).
-            const int reach = q_pos - k0 - 32 * kt0 - 4 * h;
             const int behind = window > 0 ? reach - window : -(1 << 30);
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
@@ -814,8 +827,15 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
             }
         return;
     }
-    const float total = lsum;
-    const float inv = total > 0.f ? 1.f / total : 0.f;
+    float total = lsum, stays = 1.f;
+    if (sinks != nullptr) {
+        // a sink: one more term of the denominator, unscaled, with no value behind it
+        const float sk = sinks[q_head] * 1.4426950408889634f;
+        const float top = fmaxf(m * scale_log2e, sk);
+        stays = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m * scale_log2e - top);
+        total = lsum * stays + __builtin_amdgcn_exp2f(sk - top);
+    }
+    const float inv = total > 0.f ? stays / total : 0.f;
     bf16_t* orow = out + (static_cast<size_t>(row0 + wq) * nq + q_head) * d;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -844,7 +864,7 @@ paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const f
                                           bf16_t* __restrict__ out, const int* __restrict__ q_start,
                                           const int* __restrict__ q_len, const int* __restrict__ ctx_len,
                                           int short_limit, int num_seqs, int nq, int d, int splits, int total_rows,
-                                          int grouped) {
+                                          int grouped, const float* __restrict__ sinks) {
     const int quads = d / 4, rows = blockDim.x / quads;
     const int r = blockIdx.x * rows + threadIdx.x / quads;
     const int head = blockIdx.y;
@@ -896,7 +916,14 @@ paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const f
         sum = fmaf(ls[sp], ms[sp], sum);
         a += os[sp] * ms[sp];
     }
-    const float inv = sum > 0.f ? 1.f / sum : 0.f;
+    float keep = 1.f;
+    if (sinks != nullptr) {
+        const float sk = sinks[head] * 1.4426950408889634f;
+        const float top = fmaxf(big, sk);
+        keep = big == -INFINITY ? 0.f : exp2f(big - top);
+        sum = sum * keep + exp2f(sk - top);
+    }
+    const float inv = sum > 0.f ? keep / sum : 0.f;
     ap_u32x2 w;
     w.v[0] = ap_pack2(a[0] * inv, a[1] * inv);
     w.v[1] = ap_pack2(a[2] * inv, a[3] * inv);
@@ -908,7 +935,7 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
                           const int* ctx_len, int short_limit, int num_seqs, int max_q_len, const int* block_table,
                           int max_blocks, int block_size, const void* k_pool, const void* v_pool, int nq, int nkv,
                           int d, float scale, int window, int splits, float* part_acc, float* part_ml,
-                          int total_rows, int short_rows, hipStream_t stream) {
+                          int total_rows, int short_rows, const float* sinks, const float* slopes, hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
     const size_t tile_bytes = FEED == 2 ? (2 * ap_direct_ahead(GR) + 3) * static_cast<size_t>(AP_BN) * DP * 2
@@ -944,14 +971,14 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles,
         num_seqs, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, static_cast<int>(total),
-        splits, part_acc, part_ml, compact);
+        splits, part_acc, part_ml, compact, sinks, slopes);
     PL_CHECK_LAUNCH("paged_attention_prefill");
     if (splits > 1) {
         const int rows = 256 / (d / 4);
 #define AP_MERGE(SP)                                                                                               \
     paged_attention_prefill_merge_kernel<SP><<<dim3(pl_ceil_div(total_rows, rows), nq), 256, 0, stream>>>(         \
         part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, num_seqs, nq, d, splits, \
-        total_rows, GR ? 1 : 0)
+        total_rows, GR ? 1 : 0, sinks)
         if (splits <= 2) AP_MERGE(2);
         else if (splits <= 4) AP_MERGE(4);
         else if (splits <= 8) AP_MERGE(8);
@@ -967,11 +994,11 @@ static int ap_dispatch(bool small, bool uniform_pages, const void* q, int q_stri
                        const int* q_len, const int* ctx_len, int short_limit, int num_seqs, int max_q_len,
                        const int* block_table, int max_blocks, int block_size, const void* k_pool, const void* v_pool,
                        int nq, int nkv, int d, float scale, int window, int splits, float* part_acc, float* part_ml,
-                       int total_rows, hipStream_t stream) {
+                       int total_rows, const float* sinks, const float* slopes, hipStream_t stream) {
 #define AP_LAUNCH(NW, KS, FEED)                                                                                    \
     launch_prefill<D, NW, KS, FEED>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,    \
                                     block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, \
-                                    splits, part_acc, part_ml, total_rows, 0, stream)
+                                    splits, part_acc, part_ml, total_rows, 0, sinks, slopes, stream)
     constexpr bool can_fit = 64 % (4 * D) == 0;
     constexpr int BEST = (D == 2 || D == 4) && AP_KS == 2 && AP_SMALL_KS == 2 ? AP_FEED : 1;   // the feed with uniform pages
     if constexpr (D <= 4) {
@@ -1011,7 +1038,7 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
                                           int max_q_len, const int* block_table, int max_blocks, int block_size,
                                           const void* k_pool, const void* v_pool, int nq, int nkv, int d,
                                           float scale, int window, int splits, float* part_acc, float* part_ml,
-                                          int total_rows, hipStream_t stream) {
+                                          int total_rows, const float* sinks, const float* slopes, hipStream_t stream) {
     PL_REQUIRE(splits >= 1 && splits <= AP_MERGE_MAX && (splits == 1 || (part_acc && part_ml)),
                "prefill attention: %d splits%s", splits, splits > 1 ? " without a workspace" : "");
     PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "prefill attention: head size %d, which has to be a multiple of 16 up to 256", d);
@@ -1020,6 +1047,7 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
                "prefill attention: block size %d, %d blocks a row, query stride %d, window %d", block_size, max_blocks,
                q_stride, window);
     PL_REQUIRE((nkv * d) % 8 == 0, "prefill attention: a cache row of %d elements is not read 16 bytes at a time", nkv * d);
+    PL_REQUIRE(slopes == nullptr || scale != 0.f, "prefill attention: distance slopes with a scale of zero");
     if (num_seqs <= 0 || max_q_len <= 0) return 0;
     PL_REQUIRE(total_rows >= max_q_len, "prefill attention: %d rows for a portion of %d", total_rows, max_q_len);
     PL_REQUIRE(static_cast<unsigned long long>(block_size) * nkv * d * 2 < (1ull << 32),
@@ -1037,7 +1065,7 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
 #define AP_CALL(D)                                                                                                 \
     return ap_dispatch<D>(small, pages_fit, q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
                           block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, splits,   \
-                          part_acc, part_ml, total_rows, stream)
+                          part_acc, part_ml, total_rows, sinks, slopes, stream)
     switch (dt) {
         case 1: AP_CALL(1);
         case 2: AP_CALL(2);
@@ -1069,7 +1097,8 @@ extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out
                                           int max_q_len, const int* block_table, int max_blocks, int block_size,
                                           const void* k_pool, const void* v_pool, int nq, int nkv, int d,
                                           float scale, int window, int splits, float* part_acc, float* part_ml,
-                                          int total_rows, int short_rows, hipStream_t stream) {
+                                          int total_rows, int short_rows, const float* sinks, const float* slopes,
+                                          hipStream_t stream) {
     PL_REQUIRE(pl_paged_attention_grouped_applies(nq, nkv, d, block_size),
                "grouped attention: %d query heads over %d key heads of %d, pages of %d", nq, nkv, d, block_size);
     PL_REQUIRE(splits >= 1 && splits <= AP_MERGE_MAX && (splits == 1 || (part_acc && part_ml)),
@@ -1083,8 +1112,8 @@ extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out
     if (d == 64)
         return launch_prefill<2, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
                                                 block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,
-                                                window, splits, part_acc, part_ml, total_rows, short_rows, stream);
+                                                window, splits, part_acc, part_ml, total_rows, short_rows, sinks, slopes, stream);
     return launch_prefill<4, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
                                             block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,
-                                            window, splits, part_acc, part_ml, total_rows, short_rows, stream);
+                                            window, splits, part_acc, part_ml, total_rows, short_rows, sinks, slopes, stream);
 }

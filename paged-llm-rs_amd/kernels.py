@@ -54,9 +54,9 @@ def _signatures(lib) -> None:
         "pl_gemm_stream_splits": [i, i, i, i],
         "pl_gemm_finish": [p, p, ctypes.c_longlong, i, i, i, i, i, p],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, i, f, i, i,
-                                      i, p, p, i, f, p, p, i, p],
-        "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
-        "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, i, p],
+                                      i, p, p, i, f, p, p, i, p, p, p],
+        "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p, p, p],
+        "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, i, p, p, p],
         "pl_paged_attention_grouped_applies": [i, i, i, i],
         "pl_recurrent_scan": [i, p, i, i, i, i, p, i, i, i, p, p, f, p, ctypes.c_long, i, i, i, p, p, p, p,
                               i, i, i, i, i, i, p],
@@ -412,14 +412,17 @@ def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
                            k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int, scale: float,
                            window: int = 0, splits: int = 1, q_len: torch.Tensor | None = None,
                            short_limit: int = 0, fuse: "QkFusion | None" = None, live_seqs: int | None = None,
-                           short_rows: int = 0) -> torch.Tensor:
+                           short_rows: int = 0, sinks: torch.Tensor | None = None,
+                           slopes: torch.Tensor | None = None) -> torch.Tensor:
     """bfloat16 attention of single tokens over their requests' pages, split along the context.
     With ``q_len`` the tokens of requests with ``short_limit`` tokens or more are left out; ``short_rows``
     then bounds the tokens that the other requests bring (0: not known) and ``live_seqs`` says how many
     requests, the first ones, bring tokens, so that the launch has workgroups for those tokens only.
     With ``fuse`` the rows of ``q`` are the raw projection [q | k | v]: queries (and, when it says so, each
-    token's key) are normalised and rotated inside the kernel, and key and value are written into the pages."""
+    token's key) are normalised and rotated inside the kernel, and key and value are written into the pages.
+    ``sinks`` and ``slopes``: as in ``paged_attention_plain``."""
     n = positions.numel()
+    sinks, slopes = _head_numbers(sinks, "sinks", nq), _head_numbers(slopes, "distance slopes", nq)
     _need(q, "query buffer", None, torch.bfloat16)
     if q.dim() != 2 or q.shape[0] != n or q.shape[1] != q_row_stride or q_row_stride < nq * d:
         raise TensorError(f"query buffer has shape {tuple(q.shape)} for {n} tokens and row stride {q_row_stride}")
@@ -460,7 +463,8 @@ def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
         int(block_table.shape[0] if live_seqs is None else live_seqs), int(short_rows if q_len is not None else 0),
         block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), n, nq, nkv, d, float(scale), int(window or 0), int(splits),
-        mode, _ptr(q_gain), _ptr(k_gain), gain_code, float(eps), _ptr(cos), _ptr(sin), int(rot), _stream()))
+        mode, _ptr(q_gain), _ptr(k_gain), gain_code, float(eps), _ptr(cos), _ptr(sin), int(rot), _ptr(sinks),
+        _ptr(slopes), _stream()))
     return out
 
 
@@ -480,7 +484,8 @@ def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
                             q_len: torch.Tensor, ctx_len: torch.Tensor, max_q_len: int, block_table: torch.Tensor,
                             block_size: int, k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int,
                             scale: float, window: int = 0, short_limit: int = 0, max_ctx: int | None = None,
-                            splits: int | None = None, live_seqs: int | None = None) -> torch.Tensor:
+                            splits: int | None = None, live_seqs: int | None = None,
+                            sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
     """bfloat16 attention of prompt portions on the matrix cores.  Request s brings the rows
     q_start[s] .. q_start[s]+q_len[s]-1 at the positions ctx_len[s]-q_len[s] .. ctx_len[s]-1;
     requests with fewer than ``short_limit`` tokens are skipped.  ``max_ctx`` (the longest context
@@ -516,7 +521,8 @@ def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
         q.data_ptr(), q_row_stride, out.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
         int(short_limit), live, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), int(splits),
-        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, n, _stream()))
+        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, n,
+        _ptr(_head_numbers(sinks, "sinks", nq)), _ptr(_head_numbers(slopes, "distance slopes", nq)), _stream()))
     return out
 
 
@@ -555,7 +561,8 @@ def paged_attention_grouped(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
                             block_size: int, k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int,
                             scale: float, window: int = 0, short_limit: int = 0, max_ctx: int | None = None,
                             splits: int | None = None, live_seqs: int | None = None,
-                            tokens: int | None = None) -> torch.Tensor:
+                            tokens: int | None = None, sinks: torch.Tensor | None = None,
+                            slopes: torch.Tensor | None = None) -> torch.Tensor:
     """bfloat16 attention for single tokens and the tokens of short portions, the query heads of a
     key-head group as the rows of a tile of the tiled kernel.  Arguments as for
     ``paged_attention_prefill``, but requests with ``short_limit`` tokens or more are the ones skipped
@@ -590,7 +597,8 @@ def paged_attention_grouped(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
         q.data_ptr(), q_row_stride, out.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
         int(short_limit), live, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), int(splits),
-        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, n, int(tokens or 0), _stream()))
+        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, n, int(tokens or 0),
+        _ptr(_head_numbers(sinks, "sinks", nq)), _ptr(_head_numbers(slopes, "distance slopes", nq)), _stream()))
     return out
 
 
@@ -649,14 +657,16 @@ TILED_TAKES_SHORT_WORKGROUPS = 512
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int,
-                    scale: float, window: int = 0) -> torch.Tensor:
+                    scale: float, window: int = 0, sinks: torch.Tensor | None = None,
+                    slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention for every token of a step.  ``qkv`` rows begin with the rotated queries.
     In bfloat16 the long portions go to the tiled kernel and the tokens of short ones
     (decoded tokens among them) to the kernel for single tokens, or, where many query heads share a key
     head, to the tiled kernel with a group's heads as its rows; all read the same pages."""
-    if qkv.dtype != torch.bfloat16 or _attention_mode != "kernel":
+    if qkv.dtype != torch.bfloat16 or _attention_mode != "kernel" or d % 16 or d > 256:
         return paged_attention_plain(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
-                                     kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window)
+                                     kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
+                                     sinks=sinks, slopes=slopes)
     stride = qkv.shape[1]
     short_tokens = batch.tokens_of_short_requests(SHORT_PORTION)
     if batch.max_q_len >= SHORT_PORTION:
@@ -668,7 +678,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
         paged_attention_prefill(qkv, stride, out, batch.q_start, batch.q_len, batch.ctx_len, batch.max_q_len,
                                 kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
                                 short_limit=0 if all_tiled else SHORT_PORTION, max_ctx=batch.max_ctx_len,
-                                live_seqs=getattr(batch, "live_seqs", None))
+                                live_seqs=getattr(batch, "live_seqs", None), sinks=sinks, slopes=slopes)
         if short_tokens == 0 or all_tiled:
             return out
     mixed = batch.max_q_len >= SHORT_PORTION
@@ -678,12 +688,14 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
                                        min(batch.max_q_len, SHORT_PORTION - 1), kv.block_table, kv.block_size,
                                        kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
                                        short_limit=SHORT_PORTION if mixed else 0, max_ctx=batch.max_ctx_len,
-                                       live_seqs=getattr(batch, "live_seqs", None), tokens=short_tokens)
+                                       live_seqs=getattr(batch, "live_seqs", None), tokens=short_tokens,
+                                       sinks=sinks, slopes=slopes)
     splits = decode_splits(short_tokens, nq, nkv, batch.max_ctx_len, d)
     return paged_attention_decode(qkv, stride, out, batch.positions, batch.seq_of, kv.block_table,
                                   kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
                                   q_len=batch.q_len if mixed else None, short_limit=SHORT_PORTION if mixed else 0,
-                                  live_seqs=getattr(batch, "live_seqs", None), short_rows=short_tokens)
+                                  live_seqs=getattr(batch, "live_seqs", None), short_rows=short_tokens,
+                                  sinks=sinks, slopes=slopes)
 
 
 class HandedNorm:
@@ -1442,6 +1454,6 @@ def add_position_rows_(x: torch.Tensor, table: torch.Tensor, positions: torch.Te
 def sink_attention(q: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int, scale: float,
                    window: int = 0, sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention for every token of a step with a sink a head in the softmax's denominator and a penalty a
-    head on the distance; ``q`` [n, nq * d] holds the prepared queries."""
-    return paged_attention_plain(q, q.shape[1], out, batch.positions, batch.seq_of, kv.block_table, kv.block_size,
-                                 kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, sinks=sinks, slopes=slopes)
+    head on the distance; ``q`` [n, nq * d] holds the prepared queries.  In bfloat16 the matrix-core kernel for
+    portions and the kernels for single tokens, for head sizes they take; the plain kernel otherwise."""
+    return paged_attention(q, out, batch, kv, nq, nkv, d, scale, window, sinks=sinks, slopes=slopes)
