@@ -1,0 +1,364 @@
+"""The Lefavik design in the engine against the plain implementation: every mixer alone, whole prompts, tokens
+decoded one by one, portions down to two tokens, mixed batches with pages used again, keys far away under a
+sharp softmax, keys just inside and just outside a window (in prompts and while decoding, at page borders),
+sinks that carry weight, the first tokens of a request, long decoding, and greedy generation through the
+engine's own entry point and the command line."""
+
+from __future__ import annotations
+
+import copy
+import json
+import random
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import lefavik_util as lu
+import replay_util as ru
+
+pytestmark = pytest.mark.gpu
+
+# Against the plain implementation (64-bit): 32-bit runs are held tightly.  In bfloat16 the rounding of q and k is
+# amplified by sharp softmaxes, so such runs get a loose bound there and a tight one against the engine's own
+# whole-prompt run of the same requests (the same roundings; what differs between schedules is the cache and the
+# batch: a lost key shows there in full).  All bounds are for a position that amplifies rounding as the median position
+# does, and grow with a position's own amplification.
+TOLERANCE = {"float32": 5e-5, "bfloat16": 0.1}
+BETWEEN_SCHEDULES = 4e-2
+DTYPES = ["float32", "bfloat16"]
+
+
+def replayer(folder, dtype, prompts, live=4, block_size=16, graphs=True):
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    return Replayer(folder, dtype, max_tokens=ru.pool_tokens(prompts, live), block_size=block_size, max_live=live,
+                    graphs=graphs)
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    made = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in made:
+            made[name, dtype] = lu.write_model(tmp_path_factory.mktemp(f"lefavik_{name}_{dtype}"), lu.CONFIGS[name],
+                                               seed=sorted(lu.CONFIGS).index(name) + 1, dtype=dtype, edit=lu.wide_sinks)
+        return made[name, dtype]
+    return get
+
+
+_whole: dict = {}
+_factor: dict = {}
+_plain: dict = {}
+
+
+def check(folder, dtype, prompts, steps, live=4, block_size=16, tolerance=None):
+    r = replayer(folder, dtype, prompts, live, block_size)
+    got = ru.collect(r, steps)
+    key = (str(folder), repr(sorted(prompts.items())))
+    if key not in _plain:
+        _plain[key] = lu.plain_logits(folder, prompts)
+        _factor[key] = lu.sensitivity(folder, prompts)
+    want, factor = _plain[key], _factor[key]
+    scale = max(float(want[n][p].abs().max()) for (n, p) in got)
+    bound = tolerance or TOLERANCE[dtype]
+    for (n, p), row in got.items():
+        ref = want[n][p].numpy()
+        assert row.shape == ref.shape
+        err = float(np.abs(row.astype(np.float64) - ref).max()) / scale
+        assert err <= bound * float(factor[n][p]), f"{err:.3e} at {(n, p)}, where the bound is {bound * float(factor[n][p]):.3e}"
+    assert r.cache.manager.live_sequences == 0, "every request's pages came back"
+    if dtype == "bfloat16":
+        if key not in _whole:
+            _whole[key] = ru.collect(replayer(folder, dtype, prompts, live), ru.whole(prompts))
+        spread = float(np.mean([want[n][p].std() for (n, p) in got]))
+        over = {}
+        for (n, p), row in got.items():
+            gap = float(np.sqrt(np.mean((row - _whole[key][(n, p)]) ** 2))) / spread
+            if gap > BETWEEN_SCHEDULES * float(factor[n][p]):
+                over[n, p] = gap / (BETWEEN_SCHEDULES * float(factor[n][p]))
+        assert len(over) <= max(1, len(got) // 50) and all(x <= 3.0 for x in over.values()), \
+            f"between this schedule and the whole prompt, over the bound by {sorted(over.items(), key=lambda x: -x[1])[:5]} of {len(got)}"
+    return r, got
+
+
+# --- every mixer alone, in 32-bit, the stream behind the layer against the plain implementation's ----------------
+
+ALONE = {
+    "latent": [lu.latent(3, 24, 8, 40, 56, 0.3, base=300.0)],
+    "latent, part of the rotated values turn": [lu.latent(2, 16, 12, 16, 20, 0.4, base=40.0, turned=6)],
+    "latent, a layer that reads another's vectors": [lu.latent(2, 16, 8, 24, 40, 0.3, base=300.0),
+                                                     lu.latent(5, 24, 8, 16, 40, 0.5, base=300.0, kv_from=0)],
+    "attention, a window and a temperature": [lu.attention(6, 3, 24, 40, 1.2, window=7, q_temp=(0.8, 4))],
+    "attention, neither": [lu.attention(2, 1, 40, 24, 0.5)],
+    "feed-forward": [lu.attention(1, 1, 16, 16, 0.5, mlp=lu.dense(136))],
+}
+
+
+@pytest.mark.parametrize("which", sorted(ALONE))
+def test_a_mixer_alone_against_its_plain_function(tmp_path, which):
+    """32-bit, the stream behind every layer against the plain implementation's: whole, and again in portions
+    (the later portions read what the earlier ones left in the pages)."""
+    config = lu.model(88, 61, ALONE[which], eps=1e-5, scale=1.3, logit_scale=0.7, max_positions=64)
+    folder = lu.write_model(tmp_path / "m", config, seed=7, std=0.2, edit=lu.wide_sinks)
+    tokens = [random.Random(3).randrange(61) for _ in range(45)]
+    cfg, weights = lu.load_plain(folder)
+    want = []
+    lu.plain.forward(cfg, weights, tokens, want)
+    layers = len(ALONE[which])
+    r = replayer(folder, "float32", {"a": tokens}, graphs=False)
+    rec = {}
+    r.step([{"id": "a", "tokens": tokens, "want": []}], ["a"], trace=rec)
+    for i in range(layers):
+        got = rec[f"l{i}.out"].double().cpu()
+        assert (got - want[i]).abs().max() <= 5e-5 * want[i].abs().max(), (which, i)
+    pieces, at = [[] for _ in range(layers)], 0
+    for n in (1, 2, 17, 3, 22):
+        rec = {}
+        r.step([{"id": "b", "tokens": tokens[at:at + n], "want": []}], ["b"] if at + n == 45 else [], trace=rec)
+        for i in range(layers):
+            pieces[i].append(rec[f"l{i}.out"].double().cpu())
+        at += n
+    for i in range(layers):
+        assert (torch.cat(pieces[i]) - want[i]).abs().max() <= 5e-5 * want[i].abs().max(), (which, i, "in portions")
+
+
+# --- whole models of other sizes under every schedule ----------------------------------------------------------------
+
+LENGTHS = [70, 3, 41, 18, 1, 33, 57]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", sorted(lu.CONFIGS))
+def test_whole_prompts(folders, name, dtype):
+    prompts = ru.make_prompts(lu.CONFIGS[name]["vocab"], LENGTHS, seed=1)
+    check(folders(name, dtype), dtype, prompts, ru.whole(prompts))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", sorted(lu.CONFIGS))
+def test_prefill_then_tokens_one_by_one(folders, name, dtype):
+    prompts = ru.make_prompts(lu.CONFIGS[name]["vocab"], LENGTHS, seed=1)
+    check(folders(name, dtype), dtype, prompts, ru.tail_decoded(prompts, tail=40))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", sorted(lu.CONFIGS))
+@pytest.mark.parametrize("block_size", [16, 8])
+def test_portions_down_to_two_tokens(folders, name, dtype, block_size):
+    prompts = ru.make_prompts(lu.CONFIGS[name]["vocab"], LENGTHS, seed=1)
+    check(folders(name, dtype), dtype, prompts, ru.portions(prompts), block_size=block_size)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", sorted(lu.CONFIGS))
+@pytest.mark.parametrize("seed", [0, 1])
+def test_unequal_requests_together_with_pages_used_again(folders, name, dtype, seed):
+    """Nine requests of unequal length through a pool that holds the four largest: portions of some beside single
+    tokens of others, requests left out of steps, pages of finished requests taken by the next."""
+    prompts = ru.make_prompts(lu.CONFIGS[name]["vocab"], [70, 3, 41, 18, 1, 33, 57, 64, 22], seed=2 + seed)
+    check(folders(name, dtype), dtype, prompts, ru.mixed(prompts, seed=seed, max_live=4, tail=14))
+
+
+def test_schedules_agree_with_each_other_in_32_bit(folders):
+    folder = folders("odd", "float32")
+    prompts = ru.make_prompts(lu.ODD["vocab"], LENGTHS, seed=1)
+    whole = ru.collect(replayer(folder, "float32", prompts), ru.whole(prompts))
+    scale = max(float(np.abs(row).max()) for row in whole.values())
+    for steps in (ru.tail_decoded(prompts, tail=40), ru.portions(prompts), ru.mixed(prompts, seed=5)):
+        for key, row in ru.collect(replayer(folder, "float32", prompts), steps).items():
+            assert float(np.abs(row - whole[key]).max()) <= 2e-5 * scale, key
+
+
+# --- keys far away, window edges, sinks ----------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_one_key_among_hundreds_under_a_sharp_softmax(tmp_path, dtype):
+    """Scales several times the usual make every softmax sharp: a position's weight lies on one or two keys, often
+    hundreds of tokens back (the latent layers see the whole prompt), so a key lost at a page border, at the edge of a
+    tile of keys or between shares of the context moves the logits in full."""
+    config = lu.model(64, 90, [lu.latent(4, 16, 16, 16, 48, 2.5, base=1000.0, mlp=lu.dense(64)),
+                               lu.attention(4, 2, 32, 32, 9.0, window=150, q_temp=(0.5, 64)),
+                               lu.latent(2, 32, 16, 32, 48, 2.0, base=1000.0, kv_from=0)], max_positions=1024)
+    folder = lu.write_model(tmp_path / "m", config, seed=11, dtype=dtype, std=0.15, edit=lu.wide_sinks)
+    prompts = ru.make_prompts(90, [700, 333], seed=4)
+    cfg, weights = lu.load_plain(folder)
+    # the test's own premise: the first layer's softmaxes are sharp and their heaviest keys lie far back
+    h = lu.plain.embed(cfg, weights, torch.tensor(prompts["r0"]), torch.arange(700))
+    h = lu.plain.rms(h, 1e-6) * weights["l0.norm1"]
+    m = cfg["layers"][0]["mixer"]
+    c, k_rot = lu.plain.latent_of(h, weights, "l0.mix.", m, 1e-6, torch.arange(700))
+    q = (h @ weights["l0.mix.q"].T).view(700, 4, 32)
+    score = (q[:, 0, :16] @ (c @ weights["l0.mix.uk"].T).view(700, 4, 16)[:, 0].T
+             + lu.plain.rotate_neighbours(q[:, 0, 16:], torch.arange(700), 16, 1000.0) @ k_rot.T) * m["scale"]
+    score = score.masked_fill(~torch.tril(torch.ones(700, 700, dtype=torch.bool)), -np.inf)
+    far = (torch.arange(700) - score.argmax(-1))[400:]
+    assert (far > 100).float().mean() > 0.3 and torch.softmax(score, -1).max(-1).values[400:].median() > 0.3
+    steps = ru.tail_decoded(prompts, tail=48)
+    for s in steps:            # every position of the long first steps is compared, and every decoded token
+        for e in s["entries"]:
+            e["want"] = list(range(0, len(e["tokens"]), 7)) + ([len(e["tokens"]) - 1] if (len(e["tokens"]) - 1) % 7 else [])
+    # (in bfloat16 the sharp softmaxes amplify the rounding of q and k many times: the bound against the plain
+    # implementation is loose there, and the one against the engine's own whole prompts is what finds a lost key)
+    loose = 0.5 if dtype == "bfloat16" else None
+    check(folder, dtype, prompts, steps, live=2, tolerance=loose)
+    check(folder, dtype, prompts, ru.portions(prompts, sizes=(130, 2, 61, 16, 17, 300, 5)), live=2, tolerance=loose)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 2, 16, 17, 33])
+def test_keys_just_inside_and_just_outside_a_window(tmp_path, dtype, window):
+    """A window layer alone whose scale is small, so that its softmax is flat and every key of the window carries its
+    share of the weight (under a sharp softmax most positions would not notice a key at the edge): the engine's logits
+    are the plain implementation's with this window, and clearly not those with a window one token larger or smaller,
+    in prompts, in portions and for tokens decoded one by one, with pages of 16 and of 4 tokens (a window's first key
+    at a page's border, before it and behind it)."""
+    config = lu.model(48, 70, [lu.attention(8, 2, 16, 16, 0.05, window=window, q_temp=(0.3, 8))], max_positions=128)
+    folder = lu.write_model(tmp_path / "m", config, seed=20 + window, dtype=dtype, std=0.25)
+    prompts = ru.make_prompts(70, [90, 49], seed=6)
+    want = lu.plain_logits(folder, prompts)
+    others = []
+    for other in (window - 1, window + 1):
+        if other >= 1:
+            changed = copy.deepcopy(config)
+            changed["layers"][0]["mixer"]["mask"]["size"] = other
+            others.append(lu.plain_logits(folder, prompts, changed))
+    for block_size in (16, 4):
+        for steps in (ru.whole(prompts), ru.tail_decoded(prompts, tail=45), ru.portions(prompts, sizes=(18, 2, 15, 33, 3))):
+            got = ru.collect(replayer(folder, dtype, prompts, live=2, block_size=block_size), steps)
+            closer = total = 0
+            for (n, p), row in got.items():
+                if p < window + 1:
+                    continue
+                err = float(np.abs(row - want[n][p].numpy()).max())
+                for o in others:
+                    total += 1
+                    closer += err < 0.25 * float((want[n][p] - o[n][p]).abs().max())
+            assert total > 10 and closer >= (total if dtype == "float32" else 0.9 * total), (block_size, closer, total)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sinks_that_carry_weight(tmp_path, dtype):
+    """Sinks between -1.5 and 2.5 beside scores of the same size: the engine agrees with the plain implementation, whose
+    logits move by far more than the engine's error when the sinks are set to zero, doubled, or taken away."""
+    config = lu.model(64, 80, [lu.latent(4, 16, 8, 16, 32, 0.3, base=100.0), lu.attention(4, 2, 16, 16, 1.0, window=20),
+                               lu.latent(8, 8, 8, 8, 32, 0.4, base=100.0, kv_from=0)], max_positions=128)
+    folder = lu.write_model(tmp_path / "m", config, seed=31, dtype=dtype, std=0.2, edit=lu.wide_sinks)
+    prompts = ru.make_prompts(80, [60, 5], seed=8)
+    _, got = check(folder, dtype, prompts, ru.tail_decoded(prompts, tail=20), live=2)
+    cfg, weights = lu.load_plain(folder)
+    want = {n: lu.plain.forward(cfg, weights, t) for n, t in prompts.items()}
+    for change in (lambda s: s * 0, lambda s: s * 2, lambda s: s - 50):
+        changed = {k: (change(v) if k.endswith(".sink") else v) for k, v in weights.items()}
+        moved = {n: lu.plain.forward(cfg, changed, t) for n, t in prompts.items()}
+        # (over all compared positions together: a single position may hardly feel one of the changes)
+        part = 0.01 if dtype == "float32" else 0.3
+        err = np.sqrt(np.mean([np.mean((row - want[n][p].numpy()) ** 2) for (n, p), row in got.items()]))
+        shift = np.sqrt(np.mean([float(((want[n][p] - moved[n][p]) ** 2).mean()) for (n, p) in got]))
+        assert err < part * shift, (err, shift)
+
+
+def test_the_first_tokens_of_a_request(folders):
+    """Requests of one, two and three tokens, whole and token by token, in slots and pages that others have just left."""
+    folder = folders("ones", "float32")
+    prompts = ru.make_prompts(lu.ONES["vocab"], [1, 2, 3, 1, 2, 3, 1], seed=9)
+    want = lu.plain_logits(folder, prompts)
+    r = replayer(folder, "float32", prompts, live=2)
+    for steps in (ru.whole(prompts), ru.tail_decoded(prompts, tail=3), ru.whole(prompts)):
+        got = ru.collect(r, steps)
+        worst, where = ru.worst_error(got, want)
+        assert worst <= 5e-5, where
+
+
+def test_long_decoding(folders):
+    """Two hundred tokens decoded one by one from captured steps, beside a second request, past windows and page
+    borders, against the plain implementation, in bfloat16 against the engine's own whole prompts as well."""
+    for dtype in DTYPES:
+        folder = folders("odd", dtype)
+        prompts = ru.make_prompts(lu.ODD["vocab"], [230, 215], seed=12)
+        steps = []
+        for name, toks in prompts.items():
+            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks[:15], "want": [14]}], "end": []})
+        for p in range(15, 230):
+            entries = [{"id": n, "tokens": [t[p]], "want": [0]} for n, t in prompts.items() if p < len(t)]
+            steps.append({"step": len(steps), "entries": entries, "end": [n for n, t in prompts.items() if p == len(t) - 1]})
+        check(folder, dtype, prompts, steps, live=2)
+
+
+# --- the engine's own entry point ----------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_greedy_generation_through_the_engine(folders, dtype):
+    """Prompts of unequal length through Engine.generate (scheduler, portions of 8 tokens, batches, captured steps,
+    steps queued ahead) against greedy decoding with the plain implementation."""
+    from paged_llm_rs_amd import Engine
+
+    folder = folders("odd", "float32" if dtype == "f32" else "bfloat16")
+    prompts = list(ru.make_prompts(lu.ODD["vocab"], [5, 23, 1, 40, 12, 9], seed=10).values())
+    engine = Engine(folder, dtype=dtype, block_size=16, num_blocks=24, max_batch=4, chunk=8)
+    got = engine.generate(prompts, max_tokens=12, temperature=0.0, stop_tokens=[])
+    if dtype == "f32":
+        for prompt, result in zip(prompts, got):
+            assert result["tokens"] == lu.plain_greedy(folder, prompt, 12), prompt
+    else:
+        cfg, weights = lu.load_plain(folder)
+        for prompt, result in zip(prompts, got):
+            logits = lu.plain.forward(cfg, weights, prompt + result["tokens"])[len(prompt) - 1:-1]
+            chosen = logits[torch.arange(12), torch.tensor(result["tokens"])]
+            assert (logits.max(-1).values - chosen).max() <= 0.05 * logits.abs().max(), prompt
+    assert engine.cache.manager.live_sequences == 0
+
+
+def test_requests_that_give_way_are_computed_again(folders):
+    """A pool too small for all residents: the newest gives way, comes back and recomputes its prompt; the tokens are
+    those of an engine with room to spare."""
+    from paged_llm_rs_amd import Engine
+
+    folder = folders("odd", "float32")
+    prompts = list(ru.make_prompts(lu.ODD["vocab"], [30, 28, 26, 31], seed=13).values())
+    roomy = Engine(folder, dtype="f32", block_size=8, num_blocks=64, max_batch=4, chunk=16)
+    want = roomy.generate(prompts, max_tokens=24, temperature=0.0, stop_tokens=[])
+    tight = Engine(folder, dtype="f32", block_size=8, num_blocks=19, max_batch=4, chunk=16)
+    got = tight.generate(prompts, max_tokens=24, temperature=0.0, stop_tokens=[])
+    assert sum(r["preemptions"] for r in got) > 0, "the pool was meant to run dry"
+    assert [r["tokens"] for r in got] == [r["tokens"] for r in want]
+
+
+def test_the_trace_runner_and_the_command_line_run_the_design(tmp_path):
+    folder = lu.write_model(tmp_path / "m", lu.ODD, seed=2, dtype="bfloat16")
+    repo = Path(__file__).resolve().parent.parent
+    prompts = ru.make_prompts(lu.ODD["vocab"], [20, 9], seed=3)
+    steps = ru.mixed(prompts, seed=1, max_live=2, tail=4)
+    out = tmp_path / "out"
+    done = subprocess.run([sys.executable, str(repo / "bin" / "trace_run"), "--model", str(folder), "--dtype", "float32",
+                           "--out", str(out), "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                          capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert [line for line in done.stdout.splitlines() if line.startswith("done ")] == [f"done {s['step']}" for s in steps]
+    want = lu.plain_logits(folder, prompts)
+    fed: dict = {}
+    for s in steps:
+        rows = [(e["id"], fed.get(e["id"], 0) + w) for e in s["entries"] for w in e["want"]]
+        for e in s["entries"]:
+            fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
+        if rows:
+            got = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(len(rows), -1)
+            for row, (n, p) in zip(got, rows):
+                assert np.abs(row - want[n][p].numpy()).max() <= 1e-4 * float(want[n][p].abs().max())
+
+
+def test_the_command_line_generates_with_the_design(tmp_path):
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(lu.ONES))
+    root = Path(__file__).resolve().parent.parent
+    done = subprocess.run([sys.executable, str(root / "bin" / "pagedllm"), "--model", str(tmp_path / "m"), "--random-weights",
+                           str(config), "--dtype", "bf16", "--prompt-ids", "1,2,3,4,5", "--prompt-ids", "9,8",
+                           "--max-tokens", "5", "--temperature", "0", "--stop-ids", ""],
+                          capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-2000:]
+    lines = [json.loads(x) for x in done.stdout.splitlines() if x.startswith("{")]
+    assert len(lines) == 2 and all(len(x["tokens"]) == 5 for x in lines), done.stdout
