@@ -301,9 +301,35 @@ def papivik_config(width: int, ff: int, heads: int, layers: int, vocab: int) -> 
             "layers": [kinds[i % 3] for i in range(layers)]}
 
 
-def papivik_table(torch, args) -> int:
-    """Prefill of 2,048 tokens and decode at batch 8 and 64 from 512-token contexts, for the Papivik design and for
-    Qwen3 dense at the same width, layers and vocabulary; one JSON line."""
+# --only lefavik: the Lefavik design (layers that keep one small vector a token and rebuild every head's keys and values
+# from it, one of them reading an earlier layer's vectors, and layers of windowed attention with sinks, distance
+# penalties and a query temperature; one norm a layer for the mixer and a gated feed-forward) at the same sizes.  The
+# pages' rows are 256 values (a vector of 192 and a rotated part of 64), the most the matrix-core attention kernels take.
+def lefavik_config(width: int, ff: int, heads: int, layers: int, vocab: int) -> dict:
+    mlp = {"kind": "dense", "ff": ff}
+
+    def latent(kv_from=None):
+        m = {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 128 ** -0.5,
+             "rot": {"dims": 64, "base": 1000000.0}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+    windowed = {"type": "attention", "mixer": {"heads": heads, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 0.5,
+                                               "mask": {"size": 512}, "q_temp": {"coef": 0.1, "every": 256}}, "mlp": mlp}
+    chosen = []
+    for i in range(layers):
+        chosen.append([latent(), windowed, latent(kv_from=i - 2)][i % 3])
+    return {"architecture": "Lefavik", "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "vocab": vocab, "width": width,
+            "logit_scale": 1.0, "max_positions": 8192, "layers": chosen}
+
+
+DESIGNS = {"papivik": papivik_config, "lefavik": lefavik_config}
+
+
+def papivik_table(torch, args, design: str = "papivik") -> int:
+    """Prefill of 2,048 tokens and decode at batch 8 and 64 from 512-token contexts, for a design of this package and
+    for Qwen3 dense at the same width, layers and vocabulary; one JSON line."""
     from paged_llm_rs_amd import write_random_model
     from paged_llm_rs_amd.cache import PagedCache
     from paged_llm_rs_amd.engine.batch import StepEntry
@@ -317,7 +343,7 @@ def papivik_table(torch, args) -> int:
             continue
         vocab = COMMON["vocab_size"]
         qwen = dict(SHAPES[beside][1], num_hidden_layers=layers, tie_word_embeddings=False)
-        for name, config in (("papivik", papivik_config(width, ff, heads, layers, vocab)), ("qwen3", qwen)):
+        for name, config in ((design, DESIGNS[design](width, ff, heads, layers, vocab)), ("qwen3", qwen)):
             with tempfile.TemporaryDirectory() as tmp:
                 say(f"{size}: writing and loading a random {layers}-layer {name} model of width {width}")
                 folder = write_random_model(Path(tmp) / "model", config, seed=0, std=0.02, gain_std=0.1, dtype="bfloat16")
@@ -351,7 +377,7 @@ def papivik_table(torch, args) -> int:
             import gc
             gc.collect()
             torch.cuda.empty_cache()
-    print(json.dumps({"papivik_beside_qwen3": out, "layers": {k: v[4] for k, v in PAPIVIK_SIZES.items()},
+    print(json.dumps({f"{design}_beside_qwen3": out, "layers": {k: v[4] for k, v in PAPIVIK_SIZES.items()},
                       "context": context, "dtype": "bf16", "data": "synthetic"}), flush=True)
     return 0
 
@@ -428,8 +454,8 @@ def main() -> int:
     parser.add_argument("--ahead", choices=["on", "off"], default="on",
                         help="--only engine: whether the engine queues a decoding step before it has read the tokens "
                              "of the one before")
-    parser.add_argument("--size", choices=sorted(PAPIVIK_SIZES), default=None, help="--only papivik: one of its sizes alone")
-    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products", "papivik"], default=None,
+    parser.add_argument("--size", choices=sorted(PAPIVIK_SIZES), default=None, help="--only papivik or lefavik: one of the sizes alone")
+    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products", "papivik", "lefavik"], default=None,
                         help="run one part alone: the decode steps at --batch, the prefill, or (not part of the "
                              "default line) the whole engine on 1/4/16/32/64/128 requests at once, 16 prompt tokens and "
                              "128 generated each, as the reference's own table of clients does; mixed: one step of a "
@@ -439,7 +465,7 @@ def main() -> int:
                              "products: the layer products of the 8B and 32B shapes at 8 to 64 rows, weights from memory, "
                              "by the library and by the two hand-written products of few rows; papivik: prefill and decode "
                              "of the Papivik design at layer sizes of the 0.6B and 8B shapes beside Qwen3 dense of the same "
-                             "width, layers and vocabulary")
+                             "width, layers and vocabulary; lefavik: the same for the Lefavik design")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")
@@ -449,8 +475,8 @@ def main() -> int:
 
     if args.only == "products":
         return products_table(torch)
-    if args.only == "papivik":
-        return papivik_table(torch, args)
+    if args.only in DESIGNS:
+        return papivik_table(torch, args, args.only)
 
     from paged_llm_rs_amd.engine.batch import StepEntry
     from paged_llm_rs_amd.engine.step import commit_step, require_gpu, run_step

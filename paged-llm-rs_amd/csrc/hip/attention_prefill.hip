@@ -1086,10 +1086,37 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
 // that are served.  Heads of 64 or 128, groups of up to 32, pages of a power of two of at least
 // 64 / (head size / 8) tokens; pl_paged_attention_grouped_applies says whether a shape is served.
 // short_rows: the most tokens that the requests served bring together (0: not known, the step's rows then).
-extern "C" int pl_paged_attention_grouped_applies(int nq, int nkv, int d, int block_size) {
-    if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 32 || (d != 64 && d != 128)) return 0;
+// (Heads of 64 and 128 over pages that the direct feed takes: two waves a workgroup, tiles straight into LDS.  Any other
+// head size that is a multiple of 16 up to 256, and any other page size: four waves a workgroup that feed LDS through
+// their registers as the token tiles of such heads do, the first wave holding the group's heads.)
+static bool ap_grouped_direct(int d, int block_size) {
+    if (d != 64 && d != 128) return false;
     const int rows_a_load = 64 / (d / 8);
-    return block_size >= rows_a_load && (block_size & (block_size - 1)) == 0 ? 1 : 0;
+    return block_size >= rows_a_load && (block_size & (block_size - 1)) == 0;
+}
+
+extern "C" int pl_paged_attention_grouped_applies(int nq, int nkv, int d, int block_size) {
+    if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 32 || block_size <= 0) return 0;
+    return d > 0 && d <= 256 && d % 16 == 0 ? 1 : 0;
+}
+
+template <int D>
+static int ap_dispatch_grouped(bool uniform_pages, const void* q, int q_stride, void* out, const int* q_start,
+                               const int* q_len, const int* ctx_len, int short_limit, int num_seqs, int max_q_len,
+                               const int* block_table, int max_blocks, int block_size, const void* k_pool,
+                               const void* v_pool, int nq, int nkv, int d, float scale, int window, int splits,
+                               float* part_acc, float* part_ml, int total_rows, int short_rows, const float* sinks,
+                               const float* slopes, hipStream_t stream) {
+#define AP_GROUPED(FEED)                                                                                           \
+    launch_prefill<D, 4, 1, FEED, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
+                                        block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,    \
+                                        window, splits, part_acc, part_ml, total_rows, short_rows, sinks, slopes, stream)
+    constexpr bool can_fit = 64 % (4 * D) == 0;
+    if constexpr (can_fit) {
+        if (uniform_pages) return AP_GROUPED(1);
+    }
+    return AP_GROUPED(0);
+#undef AP_GROUPED
 }
 
 extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out, const int* q_start,
@@ -1109,6 +1136,27 @@ extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out
     PL_REQUIRE(total_rows >= max_q_len, "grouped attention: %d rows for portions of %d", total_rows, max_q_len);
     PL_REQUIRE(static_cast<unsigned long long>(block_size) * nkv * d * 2 < (1ull << 32),
                "grouped attention: a page of %d tokens of %d heads of %d takes more bytes than 32 bits count", block_size, nkv, d);
+    PL_REQUIRE((nkv * d) % 8 == 0, "grouped attention: a cache row of %d elements is not read 16 bytes at a time", nkv * d);
+    PL_REQUIRE(slopes == nullptr || scale != 0.f, "grouped attention: distance slopes with a scale of zero");
+    if (!ap_grouped_direct(d, block_size)) {
+        const int dt = pl_ceil_div(d, 32);
+        const bool pages_fit = (block_size & (block_size - 1)) == 0 && block_size * 4 * dt >= 64 && 64 % (4 * dt) == 0;
+#define AP_CALL(D)                                                                                                 \
+    return ap_dispatch_grouped<D>(pages_fit, q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
+                                  block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window,  \
+                                  splits, part_acc, part_ml, total_rows, short_rows, sinks, slopes, stream)
+        switch (dt) {
+            case 1: AP_CALL(1);
+            case 2: AP_CALL(2);
+            case 3: AP_CALL(3);
+            case 4: AP_CALL(4);
+            case 5: AP_CALL(5);
+            case 6: AP_CALL(6);
+            case 7: AP_CALL(7);
+            default: AP_CALL(8);
+        }
+#undef AP_CALL
+    }
     if (d == 64)
         return launch_prefill<2, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
                                                 block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,

@@ -1020,6 +1020,13 @@ GROUPED_CASES = [
     (16, 2, 64, 256, [(700, 3)], 100),
     # contexts around the edges of the 64-key tiles, through more tiles than the rings of LDS buffers hold
     (64, 8, 128, 16, [(63, 1), (127, 1), (128, 1), (191, 1), (192, 1), (193, 1), (384, 1), (385, 1), (449, 2)], 0),
+    # other head sizes and pages that the direct feed does not take: four waves feed LDS through their registers
+    (16, 1, 256, 16, [(513, 1), (40, 2), (1, 1)], 0),
+    (8, 1, 160, 16, [(300, 3), (64, 1), (129, 15)], 0),
+    (24, 3, 96, 8, [(200, 1), (65, 4)], 40),
+    (16, 2, 48, 24, [(150, 2), (90, 1)], 0),
+    (32, 2, 128, 2, [(97, 1), (130, 2)], 0),
+    (9, 1, 224, 32, [(260, 1), (33, 5)], 100),
 ]
 
 
@@ -1066,10 +1073,10 @@ def test_grouped_attention_refuses_what_it_does_not_serve():
     from paged_llm_rs_amd import kernels
 
     applies = kernels.library().pl_paged_attention_grouped_applies
-    assert not applies(16, 8, 96, 16)      # a head that is neither 64 nor 128
     assert not applies(66, 2, 128, 16)     # more heads a group than a tile has rows
-    assert not applies(32, 8, 128, 2)      # pages smaller than one load of a wave
-    assert not applies(32, 8, 128, 24)     # no power of two
+    assert not applies(16, 2, 40, 16)      # a head that is no multiple of 16
+    assert not applies(16, 2, 272, 16)     # a head of more than 256
+    assert applies(16, 8, 96, 16) and applies(32, 8, 128, 2) and applies(32, 8, 128, 24)   # through the register feed
     assert not kernels.grouped_applies(32, 8, 128, 16)   # four heads a key: the vector kernel is as fast
     assert kernels.grouped_applies(64, 8, 128, 16)
 
@@ -1557,3 +1564,70 @@ def test_a_norm_handed_forward_from_one_product_to_the_next(n, H, deep, N2, swig
     if n <= 32 and N2 <= 32768:
         own = kernels.gemm_skinny(stream, w_next, torch.bfloat16, swiglu=swiglu, norm_gain=gain, eps=eps)
         assert rel(got, own.double()) < 1e-2
+
+
+SINK_CASES = [
+    # nq, nkv, d, block size, [(context length after the step, tokens of the step)], window
+    (4, 2, 48, 16, [(300, 40), (136, 1), (137, 1), (20, 20), (5, 2)], 136),      # token tiles and single tokens, a window
+    (8, 1, 160, 16, [(513, 1), (260, 130), (64, 3)], 0),                         # a group of eight heads over rows of 160
+    (16, 1, 256, 16, [(700, 1), (300, 64), (33, 2)], 0),                         # rows of 256
+    (16, 2, 128, 16, [(900, 2), (130, 1), (257, 129)], 0),                       # the grouped kernel's direct feed
+    (6, 3, 64, 8, [(77, 1), (200, 33)], 50),
+]
+
+
+@pytest.mark.parametrize("splits", [None, 1, 3])
+@pytest.mark.parametrize("nq,nkv,d,bs,requests,window", SINK_CASES)
+def test_sinks_and_distance_slopes_in_every_attention_kernel(nq, nkv, d, bs, requests, window, splits):
+    """A sink a head in the softmax's denominator and a penalty a head on the distance: the matrix-core kernel for
+    portions, the grouped kernel and the kernel for single tokens (with their merges) against the plain kernel in
+    32-bit over the same pages, and the plain kernel against 64-bit arithmetic."""
+    from paged_llm_rs_amd import kernels
+
+    ctx_lens = [c for c, _ in requests]
+    bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, torch.bfloat16, seed=nq + d + bs)
+    give_back_pages_behind_the_window(bt, k_pool, v_pool, bs, requests, window)
+    n = sum(c for _, c in requests)
+    q = (torch.randn(n, nq * d, device=DEV) * 0.7).to(torch.bfloat16)
+    q_start, q_len, positions, seq_of = [], [], [], []
+    for s, (ctx, count) in enumerate(requests):
+        q_start.append(len(positions))
+        q_len.append(count)
+        positions += list(range(ctx - count, ctx))
+        seq_of += [s] * count
+    as_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    scale = 1.3 / math.sqrt(d)
+    sinks = torch.linspace(-2.0, 3.0, nq, device=DEV)
+    slopes = torch.tensor([2.0 ** (-6.0 * (h + 1) / nq) for h in range(nq)], device=DEV)
+    g = nq // nkv
+    # the plain kernel, 32-bit copies of the same numbers, against 64-bit arithmetic
+    plain = torch.empty((n, nq * d), dtype=torch.float32, device=DEV)
+    kernels.paged_attention_plain(q.float(), nq * d, plain, as_i32(positions), as_i32(seq_of), bt, bs, k_pool.float(),
+                                  v_pool.float(), nq, nkv, d, scale, window, sinks=sinks, slopes=slopes)
+    for i in range(0, n, 7):
+        s, p = seq_of[i], positions[i]
+        first = max(0, p + 1 - window) if window else 0
+        qi = q[i].double().cpu().reshape(nq, d)
+        for h in range(nq):
+            k, v = keys[s][first:p + 1, h // g].double(), values[s][first:p + 1, h // g].double()
+            score = (k @ qi[h]) * scale - float(slopes[h]) * (p - torch.arange(first, p + 1, dtype=torch.float64))
+            top = max(float(score.max()), float(sinks[h]))
+            w = torch.exp(score - top)
+            want = (w @ v) / (w.sum() + math.exp(float(sinks[h]) - top))
+            assert rel(plain[i].reshape(nq, d)[h], want) < 1e-5, (i, h)
+    # the bfloat16 kernels, as a step would call them: portions of 16 tokens or more tiled, the others a kernel of their own
+    out = torch.full((n, nq * d), 7.0, dtype=torch.bfloat16, device=DEV)
+    limit = kernels.SHORT_PORTION
+    args = (bt, bs, k_pool, v_pool, nq, nkv, d, scale, window)
+    if max(q_len) >= limit:
+        kernels.paged_attention_prefill(q, nq * d, out, as_i32(q_start), as_i32(q_len), as_i32(ctx_lens), max(q_len), *args,
+                                        short_limit=limit, max_ctx=max(ctx_lens), splits=splits, sinks=sinks, slopes=slopes)
+    short = [c for c in q_len if c < limit]
+    if kernels.grouped_applies(nq, nkv, d, bs):
+        kernels.paged_attention_grouped(q, nq * d, out, as_i32(q_start), as_i32(q_len), as_i32(ctx_lens), max(short), *args,
+                                        short_limit=limit, max_ctx=max(ctx_lens), splits=splits, sinks=sinks, slopes=slopes)
+    else:
+        kernels.paged_attention_decode(q, nq * d, out, as_i32(positions), as_i32(seq_of), *args, splits=splits or 2,
+                                       q_len=as_i32(q_len), short_limit=limit, sinks=sinks, slopes=slopes)
+    for i in range(n):
+        assert rel(out[i].float(), plain[i]) < 1.5e-2, f"token {i} (request {seq_of[i]}, position {positions[i]})"
