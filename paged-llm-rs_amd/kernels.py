@@ -546,14 +546,16 @@ def grouped_applies(nq: int, nkv: int, d: int, block_size: int) -> bool:
     return nq >= GROUPED_FROM * nkv and bool(library().pl_paged_attention_grouped_applies(nq, nkv, d, block_size))
 
 
-def grouped_splits(tokens: int, nkv: int, max_ctx: int) -> int:
+def grouped_splits(tokens: int, nkv: int, max_ctx: int, d: int = 128) -> int:
     """Into how many shares the keys of a token are cut for the grouped kernel: two workgroups a compute
     unit (as many as its LDS holds) if the tokens and key heads alone do not give that many, every share
     two tiles of keys at least.  (Context 4,096 over 8 key heads: 16 tokens take 65 us in four shares and
-    67 in two, 8 tokens 39 us in eight shares and 41 in four.)"""
+    67 in two, 8 tokens 39 us in eight shares and 41 in four.)  Heads above 128 leave LDS room for one
+    workgroup a compute unit, and that is what their shares fill."""
     base = max(tokens * nkv, 1)
     key_tiles = -(-max(max_ctx, 1) // 64)
-    return max(1, min(16, key_tiles // 2, -(-2 * compute_units() // base)))
+    a_unit = 2 if d <= 128 else 1
+    return max(1, min(16, key_tiles // 2, -(-a_unit * compute_units() // base)))
 
 
 def paged_attention_grouped(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, q_start: torch.Tensor,
@@ -588,7 +590,7 @@ def paged_attention_grouped(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
     if not 0 < live <= S:
         raise TensorError(f"{live} requests with tokens of {S}")
     if splits is None:
-        splits = grouped_splits(n if tokens is None else int(tokens), nkv, int(max_ctx or 0))
+        splits = grouped_splits(n if tokens is None else int(tokens), nkv, int(max_ctx or 0), d)
     part_acc = part_ml = None
     if splits > 1:
         part_acc = torch.empty((n * nq * splits * d,), dtype=torch.float32, device=q.device)
