@@ -253,20 +253,40 @@ class SharedNormBlock:
     def first_norm(self):
         return self.norm1
 
+    def _norm_into_products(self, rows: int) -> bool:
+        """Whether the norm runs as the first stage of the two products that read it (few rows of a bfloat16
+        model, where both products are the hand-written kernel's) instead of as a kernel of its own."""
+        if self.dtype != torch.bfloat16 or not getattr(self.norm1, "fuses_into_product", False):
+            return False
+        readers = [getattr(self.mixer, "proj", None) if getattr(self.mixer, "takes_pending_norm", False) else None]
+        if self.feed_forward is not None:
+            readers.append(getattr(self.feed_forward, "gate_up_proj", None) if hasattr(self.feed_forward, "begin") else None)
+        return all(r is not None and r.bias is None and kernels.fused_norm_applies(rows, r.in_features, r.weight)
+                   and r.out_features <= kernels.FUSED_NORM_MAX_COLUMNS for r in readers)
+
     def forward(self, resid, delta, ctx):
-        # (the norm's rows are written out: two sublayers read them, and the first adds into the stream
-        # before the second runs)
-        rows = self.norm1.apply(resid, delta, self.dtype)
+        ffn = self.feed_forward
+        if delta is None and ctx.trace is None and self._norm_into_products(resid.shape[0]):
+            # Few rows: the norm is the first stage of the products that read it.  Both read the stream as the layer
+            # found it, so the feed-forward's first half runs before the mixer adds its output into the stream.
+            rows = PendingNorm(self.norm1, resid, self.dtype)
+            act = ffn.begin(rows) if ffn is not None else None
+        else:
+            # (the norm's rows are written out: two sublayers read them, and the first adds into the stream
+            # before the second runs)
+            rows, act = self.norm1.apply(resid, delta, self.dtype), None
         ctx.residual = resid
         mixed = self.mixer.forward(rows, ctx)
         ctx.residual = None
         if mixed is not None:
             kernels.residual_add(resid, mixed)
-        if self.feed_forward is not None:
-            if getattr(self.feed_forward, "fuses", False):
-                out = self.feed_forward.forward(rows, residual=resid, out_dtype=torch.float32)
+        if ffn is not None:
+            if act is not None:
+                out = ffn.finish(act, residual=resid, out_dtype=torch.float32)
+            elif getattr(ffn, "fuses", False):
+                out = ffn.forward(rows, residual=resid, out_dtype=torch.float32)
             else:
-                out = self.feed_forward.forward(rows)
+                out = ffn.forward(rows)
             if out is not None:
                 kernels.residual_add(resid, out)
         return None

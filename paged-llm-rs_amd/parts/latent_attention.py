@@ -34,6 +34,8 @@ from .sink_attention import head_sinks
 class LatentAttention:
     graph_safe = True
     short_portion = kernels.SHORT_PORTION
+    # forward takes a norm still to run in place of rows (its one product, ``proj``, reads them)
+    takes_pending_norm = True
 
     @staticmethod
     def declare(spec, hidden: int) -> list:
@@ -91,7 +93,7 @@ class LatentAttention:
         return None
 
     def forward(self, x, ctx):
-        """``x``: the normed rows.  The output comes back as 32-bit sums, or None where the output projection
+        """``x``: the normed rows, or a norm still to run.  The output comes back as 32-bit sums, or None where the output projection
         added them into ``ctx.residual`` itself."""
         batch, kv = ctx.batch, ctx.kv()
         H, D, rot, V, R, P = self.H, self.D, self.rot, self.V, self.R, self.padded

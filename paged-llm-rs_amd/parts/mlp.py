@@ -58,8 +58,16 @@ class GatedMlp:
             out = self.down_proj.forward(act)
             trace.record("down_proj.out", out)
             return out
+        return self.finish(self.begin(x), residual=residual, hand=hand, out_dtype=out_dtype)
+
+    def begin(self, x):
+        """The first half, act(gate x) * (up x): all that reads the feed-forward's input.  A layer whose mixer
+        adds into the stream that ``x`` is a norm of may run this half before the mixer and ``finish`` behind it."""
         # (few rows: the activation is the product's epilogue)
-        act = self.gate_up_proj.forward(x, swiglu=True, activation=self.activation)
+        return self.gate_up_proj.forward(x, swiglu=True, activation=self.activation)
+
+    def finish(self, act, residual: torch.Tensor | None = None, hand=None, out_dtype=None):
+        """The second half, down(act), added into ``residual`` where the product kernel can (None comes back)."""
         # (``out_dtype``: the type of what comes back where the product could not add it into the stream itself)
         return self.down_proj.forward(act, out_dtype=out_dtype, add_into=residual,
                                       hand=hand if residual is not None else None)

@@ -50,6 +50,8 @@ def head_slopes(kind, heads: int, span: float, device):
 class SinkAttention:
     graph_safe = True
     short_portion = kernels.SHORT_PORTION
+    # forward takes a norm still to run in place of rows (its one product, ``proj``, reads them)
+    takes_pending_norm = True
 
     @staticmethod
     def declare(spec, hidden: int) -> list:
@@ -93,7 +95,7 @@ class SinkAttention:
         return None
 
     def forward(self, x, ctx):
-        """``x``: the normed rows.  The output comes back as 32-bit sums, or None where the output projection
+        """``x``: the normed rows, or a norm still to run.  The output comes back as 32-bit sums, or None where the output projection
         added them into ``ctx.residual`` itself."""
         batch, kv = ctx.batch, ctx.kv()
         rows = self.proj.forward(x, out_dtype=torch.float32)

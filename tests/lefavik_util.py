@@ -60,7 +60,7 @@ ONES = model(100, 97, [
 # head, a window of 64 (page borders on both ends), layers that read vectors kept two and three layers earlier.
 LARGE = model(256, 300, [
     latent(4, 64, 64, 64, 192, 0.09, base=10000.0, mlp=dense(320)),
-    attention(16, 1, 128, 128, 2.0, window=64, q_temp=(0.5, 32)),
+    attention(16, 1, 128, 128, 0.15, window=64, q_temp=(0.5, 32)),
     latent(8, 32, 64, 48, 192, 0.1, base=10000.0, kv_from=0),
     latent(2, 128, 64, 128, 192, 0.07, base=10000.0, kv_from=0, mlp=dense(256)),
 ], eps=1e-6, scale=0.3, logit_scale=3.0)
