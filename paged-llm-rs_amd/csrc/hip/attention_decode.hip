@@ -200,7 +200,20 @@ __device__ __forceinline__ bool ad_find_row(int slot, const int* __restrict__ q_
 // at all times with nothing else between them in the queue of loads (page numbers come from LDS, so no
 // round waits behind a table lookup).  Queries and the own key are normalised and rotated while the
 // first two rounds are on their way.
-template <int LPK, int GT, int U, int WV>
+// EX: the launch has sinks or distance slopes; without them the kernel is compiled as if it knew neither, and takes
+// the arguments it always took.
+template <bool EX>
+struct ad_extras_t {
+    const float* sinks;
+    const float* slopes;
+};
+template <>
+struct ad_extras_t<false> {
+    static constexpr const float* sinks = nullptr;
+    static constexpr const float* slopes = nullptr;
+};
+
+template <int LPK, int GT, int U, int WV, bool EX = false>
 __global__ void __launch_bounds__(64 * WV)
 paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                               float* __restrict__ part_acc, float* __restrict__ part_ml,
@@ -209,8 +222,9 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
                               const int* __restrict__ block_table, int max_blocks, int block_size,
                               bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool, int nq,
                               int nkv, int d, float scale_log2e, int window, int splits, int tiles, int g,
-                              uint32_t splits_magic, ad_fuse_t fuse, const float* __restrict__ sinks,
-                              const float* __restrict__ slopes) {
+                              uint32_t splits_magic, ad_fuse_t fuse, ad_extras_t<EX> extras) {
+    const float* const sinks = extras.sinks;
+    const float* const slopes = extras.slopes;
     constexpr int KPW = PL_WAVE / LPK;  // keys a wave handles with one load
     constexpr int ROUND = WV * KPW * U;
     extern __shared__ float lds[];      // [AD_PAGES_LDS] page numbers, then [WV][GT][2] running max and sum, [WV][GT][d] accumulators
@@ -354,10 +368,13 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
         }
     }
     // (a penalty on the distance, where the layer has one: slope_h (pos - j) leaves the score, in the exponent's unit)
-    const bool tilted = slopes != nullptr;
-    float tilt[GT];
+    const bool tilted = EX && slopes != nullptr;
+    float tilt[EX ? GT : 1];
+    int round_now = 0;            // (EX) the round that `consume` is given, for the distance of its keys
+    if constexpr (EX) {
 #pragma unroll
-    for (int hq = 0; hq < GT; ++hq) tilt[hq] = tilted ? slopes[h0 + min(hq, heads - 1)] * 1.4426950408889634f : 0.f;
+        for (int hq = 0; hq < GT; ++hq) tilt[hq] = tilted ? slopes[h0 + min(hq, heads - 1)] * 1.4426950408889634f : 0.f;
+    }
     float m[GT], l[GT], acc[GT][8];
 #pragma unroll
     for (int hq = 0; hq < GT; ++hq) {
@@ -406,19 +423,20 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     // Values are taken two keys at a time: element i of both keys in one word against both probabilities
     // (rounded to bfloat16, as the matrix-core kernels round them), one instruction an element and head.
     static_assert(U % 2 == 0, "values are taken two keys at a time");
-    auto consume = [&](u32x4* kraw, u32x4* vraw, const bool* ok, int round) {
+    auto consume = [&](u32x4* kraw, u32x4* vraw, const bool* ok) {
         float s[U][GT];
-        const int base = s_begin + round * ROUND + wave * KPW * U;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const float far = static_cast<float>(pos - (base + u * KPW + sub));
 #pragma unroll
             for (int hq = 0; hq < GT; ++hq) {
                 float dot = 0.f;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) dot = ad_dot2(qp[hq].v[w], kraw[u].v[w], dot);
                 dot = key_sum<LPK>(dot) * scale_log2e;
-                if (tilted) dot = fmaf(-tilt[hq], far, dot);
+                if constexpr (EX) {
+                    if (tilted)
+                        dot = fmaf(-tilt[hq], static_cast<float>(pos - (s_begin + round_now * ROUND + wave * KPW * U + u * KPW + sub)), dot);
+                }
                 s[u][hq] = ok[u] ? dot : -INFINITY;
             }
             const uint32_t keep = ok[u] ? 0xffffffffu : 0u;
@@ -463,10 +481,12 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
         }
     };
     for (int r = 0; r < rounds; r += 2) {
-        consume(ka, va, oka, r);
+        if constexpr (EX) round_now = r;
+        consume(ka, va, oka);
         if (r + 2 < rounds) ask(r + 2, ka, va, oka);
         if (r + 1 < rounds) {
-            consume(kb, vb, okb, r + 1);
+            if constexpr (EX) round_now = r + 1;
+            consume(kb, vb, okb);
             if (r + 3 < rounds) ask(r + 3, kb, vb, okb);
         }
     }
@@ -516,13 +536,15 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
         }
         const int h = h0 + hq;
         if (splits == 1) {
-            if (sinks != nullptr) {
-                // a sink: one more term of the denominator, unscaled, with no value behind it
-                const float sk = sinks[h] * 1.4426950408889634f;
-                const float top = fmaxf(big, sk);
-                const float keep = big == -INFINITY ? 0.f : exp2f(big - top);
-                sum = sum * keep + exp2f(sk - top);
-                a *= keep;
+            if constexpr (EX) {
+                if (sinks != nullptr) {
+                    // a sink: one more term of the denominator, unscaled, with no value behind it
+                    const float sk = sinks[h] * 1.4426950408889634f;
+                    const float top = fmaxf(big, sk);
+                    const float keep = big == -INFINITY ? 0.f : exp2f(big - top);
+                    sum = sum * keep + exp2f(sk - top);
+                    a *= keep;
+                }
             }
             out[(static_cast<size_t>(t) * nq + h) * d + dd] = from_float<bf16_t>(sum > 0.f ? a / sum : 0.f);
         } else {
@@ -542,7 +564,7 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
 // invalidates a whole L2.)  One thread an output element; every load is asked for before any is used.
 #define AD_MAX_SPLITS 64
 
-template <int SP>
+template <int SP, bool EX = false>
 __global__ void __launch_bounds__(256)
 paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                              bf16_t* __restrict__ out, const int* __restrict__ positions,
@@ -587,7 +609,7 @@ paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __
         sum = fmaf(ls[s], w, sum);
         a = fmaf(as[s], w, a);
     }
-    if (sinks != nullptr) {
+    if (EX && sinks != nullptr) {
         const float sk = sinks[h] * 1.4426950408889634f;
         const float top = fmaxf(big, sk);
         const float keep = big == -INFINITY ? 0.f : exp2f(big - top);
@@ -610,27 +632,46 @@ static int launch_decode_keys(const void* q, int q_stride, void* out, float* par
     const int tiles = pl_ceil_div(g, GT);
     const size_t lds_bytes = (AD_PAGES_LDS + static_cast<size_t>(WV) * GT * 2 + static_cast<size_t>(WV) * GT * d) * sizeof(float);
     PL_REQUIRE(lds_bytes <= 160 * 1024, "decode attention: %zu bytes of LDS for head size %d", lds_bytes, d);
+    const bool extras = sinks != nullptr || slopes != nullptr;
     if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_decode_kernel<LPK, GT, U, WV>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        hipError_t e = extras ? hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_decode_kernel<LPK, GT, U, WV, true>),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes))
+                              : hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_decode_kernel<LPK, GT, U, WV, false>),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         PL_REQUIRE(e == hipSuccess, "decode attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     // rows of the grid: the step's rows, or, where fewer, the tokens that the short requests can bring
     const bool compact = q_len != nullptr && num_seqs > 0 && short_rows > 0 && short_rows < n;
     dim3 grid(nkv * tiles, compact ? short_rows : n, splits);
     PL_REQUIRE(n <= 65535 && splits <= 65535, "decode attention: %d tokens or %d splits are more than one launch covers", n, splits);
-    paged_attention_decode_kernel<LPK, GT, U, WV><<<grid, 64 * WV, lds_bytes, stream>>>(
-        static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), part_acc, part_ml, positions, seq_of,
-        q_len, short_limit, compact ? num_seqs : 0, block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool),
-        static_cast<bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles, g,
-        static_cast<uint32_t>((0x100000000ull + splits - 1) / static_cast<unsigned>(splits)), fuse, sinks, slopes);
+#define AD_LAUNCH(EX)                                                                                                  \
+    paged_attention_decode_kernel<LPK, GT, U, WV, EX><<<grid, 64 * WV, lds_bytes, stream>>>(                           \
+        static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), part_acc, part_ml, positions, seq_of,      \
+        q_len, short_limit, compact ? num_seqs : 0, block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool), \
+        static_cast<bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles, g,              \
+        static_cast<uint32_t>((0x100000000ull + splits - 1) / static_cast<unsigned>(splits)), fuse, more)
+    if (extras) {
+        const ad_extras_t<true> more{sinks, slopes};
+        AD_LAUNCH(true);
+    } else {
+        const ad_extras_t<false> more{};
+        AD_LAUNCH(false);
+    }
+#undef AD_LAUNCH
     PL_CHECK_LAUNCH("paged_attention_decode");
     if (splits > 1) {
         const dim3 mgrid = dim3(pl_ceil_div(nq * d, 256), compact ? short_rows : n);
 #define AD_MERGE(SP)                                                                                              \
-    paged_attention_merge_kernel<SP><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, static_cast<bf16_t*>(out),     \
-                                                                positions, seq_of, q_len, short_limit, nq, d,     \
-                                                                splits, n, compact ? num_seqs : 0, sinks)
+    do {                                                                                                          \
+        if (sinks != nullptr)                                                                                     \
+            paged_attention_merge_kernel<SP, true><<<mgrid, 256, 0, stream>>>(                                    \
+                part_acc, part_ml, static_cast<bf16_t*>(out), positions, seq_of, q_len, short_limit, nq, d,       \
+                splits, n, compact ? num_seqs : 0, sinks);                                                        \
+        else                                                                                                      \
+            paged_attention_merge_kernel<SP, false><<<mgrid, 256, 0, stream>>>(                                   \
+                part_acc, part_ml, static_cast<bf16_t*>(out), positions, seq_of, q_len, short_limit, nq, d,       \
+                splits, n, compact ? num_seqs : 0, nullptr);                                                      \
+    } while (0)
         if (splits <= 4) AD_MERGE(4);
         else if (splits <= 8) AD_MERGE(8);
         else if (splits <= 16) AD_MERGE(16);
