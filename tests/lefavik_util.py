@@ -138,3 +138,37 @@ def sensitivity(folder, prompts: dict) -> dict:
         moved = ((plain.forward(config, shaken, tokens) - base) ** 2).mean(-1).sqrt() / base.std()
         out[name] = torch.clamp(moved / (2 * moved.median()), min=1.0)
     return out
+
+
+def drawn_config(seed: int) -> dict:
+    """A configuration drawn from the sizes and constants a model of the design may have: any order of layers (the first
+    may be a window layer), layers that read an earlier layer's vectors, head counts from 1 to 16, groups of 1 to 8, head
+    parts from 8 to 128, vectors from 16 to 224, windows from 3 to beyond the prompts or none, with and without a
+    temperature and a feed-forward."""
+    import random
+
+    rng = random.Random(seed)
+    width = rng.choice([64, 96, 128, 192, 200])
+    layers, owners = [], []            # owners: (layer, kv_rank, rot_dim, base, turned) of latent layers that keep vectors
+    for i in range(rng.randint(3, 6)):
+        mlp = dense(rng.choice([64, 200])) if rng.random() < 0.7 else None
+        if rng.random() < 0.55:
+            heads, dim, vdim = rng.choice([1, 2, 4, 8, 12, 16]), rng.choice([8, 16, 32, 48, 64]), rng.choice([8, 16, 32, 64])
+            if owners and rng.random() < 0.4:
+                source, rank, rot, base, turned = rng.choice(owners)
+                layers.append(latent(heads, dim, rot, vdim, rank, (dim + rot) ** -0.5, base=base, turned=turned, kv_from=source, mlp=mlp))
+            else:
+                rank, rot = rng.choice([16, 32, 48, 64, 96, 112, 160, 192, 224]), rng.choice([2, 8, 16, 32, 64])
+                base = rng.choice([100.0, 10000.0, 250000.0])
+                turned = rot if rng.random() < 0.8 else max(2, rot // 2 // 2 * 2)
+                owners.append((i, rank, rot, base, turned))
+                layers.append(latent(heads, dim, rot, vdim, rank, (dim + rot) ** -0.5, base=base, turned=turned, mlp=mlp))
+        else:
+            kv_heads, group = rng.choice([1, 2, 4]), rng.choice([1, 2, 4, 8])
+            dim, vdim = rng.choice([16, 32, 48, 64, 128]), rng.choice([16, 32, 48, 64, 128])
+            window = rng.choice([None, 3, 20, 64, 100, 500])
+            q_temp = (rng.choice([0.1, 0.5, 1.0]), rng.choice([1, 7, 64])) if rng.random() < 0.7 else None
+            layers.append(attention(kv_heads * group, kv_heads, dim, vdim, rng.choice([0.5, 1.0, 2.0]) * dim ** -0.5, window=window,
+                                    q_temp=q_temp, mlp=mlp))
+    return model(width, rng.choice([101, 256, 333]), layers, eps=rng.choice([1e-6, 1e-5]), scale=rng.choice([1.0, width ** 0.5]),
+                 logit_scale=rng.choice([1.0, 0.5, 2.0]), max_positions=256)

@@ -166,6 +166,19 @@ def test_unequal_requests_together_with_pages_used_again(folders, name, dtype, s
     check(folders(name, dtype), dtype, prompts, ru.mixed(prompts, seed=seed, max_live=4, tail=14))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", range(10))
+def test_drawn_configurations(tmp_path, seed, dtype):
+    """Ten drawn models (order of layers, sizes, head counts, windows, constants; `lefavik_util.drawn_config`) under a
+    mixed schedule and whole, over pages of 16, 8 and 32 tokens."""
+    config = lu.drawn_config(100 + seed)
+    folder = lu.write_model(tmp_path / "m", config, seed=seed, dtype=dtype, std=0.1, edit=lu.wide_sinks)
+    prompts = ru.make_prompts(config["vocab"], [75, 9, 130, 33, 2], seed=seed)
+    block_size = (16, 8, 32)[seed % 3]
+    check(folder, dtype, prompts, ru.mixed(prompts, seed=seed, max_live=3, tail=20), live=3, block_size=block_size)
+    check(folder, dtype, prompts, ru.whole(prompts), live=3, block_size=block_size)
+
+
 def test_schedules_agree_with_each_other_in_32_bit(folders):
     folder = folders("odd", "float32")
     prompts = ru.make_prompts(lu.ODD["vocab"], LENGTHS, seed=1)
